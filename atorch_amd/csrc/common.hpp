@@ -1,0 +1,126 @@
+// Shared device helpers for the gfx950 FP8 MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/atorch_amd_fp8.h"
+
+namespace aamd {
+
+constexpr int kTile = 128;       // quantisation tile / block edge
+constexpr float kFp8Max = 448.f;  // largest finite e4m3fn magnitude
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short u16;
+
+// ---- error plumbing -------------------------------------------------------
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define AAMD_REQUIRE(cond, ...)      \
+  do {                               \
+    if (!(cond)) {                   \
+      aamd::set_error(__VA_ARGS__);  \
+      return AAMD_ERR_ARG;           \
+    }                                \
+  } while (0)
+
+#define AAMD_LAUNCH_CHECK(what)                              \
+  do {                                                       \
+    hipError_t e__ = hipGetLastError();                      \
+    if (e__ != hipSuccess) return aamd::hip_fail(e__, what); \
+  } while (0)
+
+// ---- scalar conversions ---------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 bits, round to nearest even (finite inputs and inf; NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// Input element loaders: 8 consecutive elements -> 8 floats.
+struct BF16 {
+  typedef u16 elem;
+};
+struct F32 {
+  typedef float elem;
+};
+
+__device__ __forceinline__ void unpack8(const v4i& raw, float* v) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    uint32_t w = (uint32_t)raw[i];
+    v[2 * i] = __uint_as_float(w << 16);
+    v[2 * i + 1] = __uint_as_float(w & 0xffff0000u);
+  }
+}
+
+// ---- 16-lane (one DPP row) max reduction: every lane of the row gets the max
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f32<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_f32<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_f32<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_f32<0x140>(v));  // row_mirror
+  return v;
+}
+
+// s = max(amax, eps) / 448 ; 0 -> 1.  IEEE division: the scale is part of the bit-exact contract.
+__device__ __forceinline__ float scale_from_amax(float amax, float eps) {
+  float s = fmaxf(amax, eps) / kFp8Max;
+  return s == 0.f ? 1.f : s;
+}
+
+// Two floats -> two e4m3fn codes in the low or high half of `old` (RNE, v_cvt_pk_fp8_f32).
+// Inputs are clamped to +-448 first: by construction |x/s| <= 448(1+2^-23), which RNE maps to
+// 448 anyway, so the clamp never changes an in-contract result but keeps the encoder away
+// from its overflow behaviour.
+template <bool HI>
+__device__ __forceinline__ int pack2_fp8(float a, float b, int old) {
+  a = __builtin_amdgcn_fmed3f(a, -kFp8Max, kFp8Max);
+  b = __builtin_amdgcn_fmed3f(b, -kFp8Max, kFp8Max);
+  return __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, HI);
+}
+
+// 8 values / one scale -> 8 codes in two dwords.  IEEE division per element.
+__device__ __forceinline__ v2i quant8(const float* v, float s) {
+  v2i o;
+  int w = pack2_fp8<false>(v[0] / s, v[1] / s, 0);
+  o[0] = pack2_fp8<true>(v[2] / s, v[3] / s, w);
+  w = pack2_fp8<false>(v[4] / s, v[5] / s, 0);
+  o[1] = pack2_fp8<true>(v[6] / s, v[7] / s, w);
+  return o;
+}
+
+__device__ __forceinline__ float amax8(const float* v) {
+  float m = fmaxf(fabsf(v[0]), fabsf(v[1]));
+#pragma unroll
+  for (int i = 2; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+  return m;
+}
+
+// Which group does padded tile `t` belong to?  tile_off[E+1] is an exclusive prefix of
+// per-group tile counts.  All threads of the block take part; returns the same g in every
+// thread (E+1 if t is beyond the last tile).  `slot` is one int of shared memory.
+__device__ __forceinline__ int find_group(const int32_t* __restrict__ tile_off, int E, int t, int* slot) {
+  if (threadIdx.x == 0) *slot = E + 1;
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    int lo = tile_off[e], hi = tile_off[e + 1];
+    if (t >= lo && t < hi) *slot = e;
+  }
+  __syncthreads();
+  return *slot;
+}
+
+}  // namespace aamd

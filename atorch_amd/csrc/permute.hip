@@ -1,0 +1,337 @@
+// Token routing kernels for gfx950: device-side router preprocess (histogram, scan, stable
+// counting sort), inverse permutation, and the fused unpermute + weighted combine.
+#include "common.hpp"
+
+namespace aamd {
+
+// ---------------------------------------------------------------------------------------
+// unpermute + combine: one workgroup per token, 16-byte gathers of the topk source rows.
+// PD: dtype of probs (AAMD_NONE / AAMD_BF16 / AAMD_F32).
+// ---------------------------------------------------------------------------------------
+constexpr int kMaxTopk = 64;
+
+template <int PD>
+__global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __restrict__ y, int64_t M, int H8,
+                                                                const int32_t* __restrict__ row_map,
+                                                                const void* __restrict__ probs, int topk,
+                                                                void* __restrict__ out) {
+  __shared__ int srow[kMaxTopk];
+  __shared__ float sprob[kMaxTopk];
+  const int64_t t = blockIdx.x;
+  if (threadIdx.x < topk) {
+    int r = row_map[t * topk + threadIdx.x];
+    if (r >= M) r = -1;
+    srow[threadIdx.x] = r;
+    float pv = 1.f;
+    if constexpr (PD == AAMD_BF16) pv = bf16_bits_to_f32(reinterpret_cast<const u16*>(probs)[t * topk + threadIdx.x]);
+    if constexpr (PD == AAMD_F32) pv = reinterpret_cast<const float*>(probs)[t * topk + threadIdx.x];
+    sprob[threadIdx.x] = pv;
+  }
+  __syncthreads();
+  const int64_t H = (int64_t)H8 * 8;
+  for (int c = threadIdx.x; c < H8; c += 256) {
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+#pragma unroll 4
+    for (int j = 0; j < topk; j++) {
+      const int r = srow[j];
+      if (r < 0) continue;
+      const v4i raw = *reinterpret_cast<const v4i*>(y + (int64_t)r * H + c * 8);
+      float v[8];
+      unpack8(raw, v);
+      const float pv = sprob[j];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        float prod = v[i];
+        if constexpr (PD == AAMD_BF16) prod = bf16_bits_to_f32(f32_to_bf16_bits(v[i] * pv));
+        if constexpr (PD == AAMD_F32) prod = v[i] * pv;
+        acc[i] += prod;
+      }
+    }
+    if constexpr (PD == AAMD_F32) {
+      float* dst = reinterpret_cast<float*>(out) + t * H + c * 8;
+      reinterpret_cast<v4f*>(dst)[0] = v4f{acc[0], acc[1], acc[2], acc[3]};
+      reinterpret_cast<v4f*>(dst)[1] = v4f{acc[4], acc[5], acc[6], acc[7]};
+    } else {
+      v4i w;
+#pragma unroll
+      for (int i = 0; i < 4; i++) w[i] = (int)(f32_to_bf16_bits(acc[2 * i]) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16));
+      *reinterpret_cast<v4i*>(reinterpret_cast<u16*>(out) + t * H + c * 8) = w;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// plain row permute: 16-byte chunks, each source row read once and written topk times
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void permute_rows_kernel(const v4i* __restrict__ x, int chunks,
+                                                           const int32_t* __restrict__ row_map, int topk,
+                                                           int64_t M_out, v4i* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < chunks; c += 256) {
+    const v4i v = x[t * chunks + c];
+    for (int j = 0; j < topk; j++) {
+      const int64_t dst = row_map[t * topk + j];
+      if (dst >= 0 && dst < M_out) out[dst * chunks + c] = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// inverse permutation
+// ---------------------------------------------------------------------------------------
+__global__ void fill_i32_kernel(int32_t* __restrict__ p, int64_t n, int32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+__global__ void invert_permutation_kernel(const int64_t* __restrict__ sorted_idx, int64_t n_perm, int64_t n_flat,
+                                          int32_t* __restrict__ row_map) {
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (j < n_perm) {
+    const int64_t f = sorted_idx[j];
+    if (f >= 0 && f < n_flat) row_map[f] = (int32_t)j;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// router preprocess: stable counting sort by expert id.
+//   chunk  = 1024 consecutive flat indices handled by one workgroup (4 rounds of 256)
+//   hist   [E][nchunk]: ids of expert e in chunk b            (kernel 1)
+//   scan   rows of hist -> exclusive prefix along chunks, row totals      (kernel 2)
+//   goff   exclusive prefix of the row totals                              (kernel 3)
+//   place  position = goff[e] + hist_prefix[e][b] + rank inside the chunk  (kernel 4)
+// ---------------------------------------------------------------------------------------
+constexpr int kChunk = 1024;
+
+template <typename ID>
+__device__ __forceinline__ int load_id(const ID* ids, int64_t i, int64_t n, int E) {
+  if (i >= n) return -1;
+  const int64_t e = (int64_t)ids[i];
+  return (e >= 0 && e < E) ? (int)e : -1;  // out-of-range ids are dropped (row_map -1)
+}
+
+template <typename ID>
+__global__ __launch_bounds__(256) void route_hist_kernel(const ID* __restrict__ ids, int64_t n, int E, int nchunk,
+                                                         int32_t* __restrict__ hist) {
+  extern __shared__ int cnt[];
+  for (int e = threadIdx.x; e < E; e += 256) cnt[e] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kChunk;
+#pragma unroll
+  for (int it = 0; it < kChunk / 256; it++) {
+    const int e = load_id(ids, base + it * 256 + threadIdx.x, n, E);
+    if (e >= 0) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) hist[(int64_t)e * nchunk + blockIdx.x] = cnt[e];
+}
+
+__global__ __launch_bounds__(256) void route_rowscan_kernel(int32_t* __restrict__ hist, int nchunk,
+                                                            int32_t* __restrict__ totals) {
+  __shared__ int buf[256];
+  __shared__ int carry;
+  int32_t* row = hist + (int64_t)blockIdx.x * nchunk;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < nchunk; base += 256) {
+    const int i = base + threadIdx.x;
+    const int v = i < nchunk ? row[i] : 0;
+    buf[threadIdx.x] = v;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+      __syncthreads();
+      buf[threadIdx.x] += t;
+      __syncthreads();
+    }
+    if (i < nchunk) row[i] = carry + buf[threadIdx.x] - v;
+    __syncthreads();
+    if (threadIdx.x == 255) carry += buf[255];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) totals[blockIdx.x] = carry;
+}
+
+__global__ __launch_bounds__(256) void route_goff_kernel(const int32_t* __restrict__ totals, int E,
+                                                         int64_t* __restrict__ goff) {
+  __shared__ int buf[256];
+  __shared__ long long carry;
+  if (threadIdx.x == 0) {
+    carry = 0;
+    goff[0] = 0;
+  }
+  __syncthreads();
+  for (int base = 0; base < E; base += 256) {
+    const int e = base + threadIdx.x;
+    buf[threadIdx.x] = e < E ? totals[e] : 0;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+      __syncthreads();
+      buf[threadIdx.x] += t;
+      __syncthreads();
+    }
+    if (e < E) goff[e + 1] = carry + buf[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 255) carry += buf[255];
+    __syncthreads();
+  }
+}
+
+template <typename ID>
+__global__ __launch_bounds__(256) void route_place_kernel(const ID* __restrict__ ids, int64_t n, int E, int nchunk,
+                                                          const int32_t* __restrict__ hist,
+                                                          const int64_t* __restrict__ goff,
+                                                          int64_t* __restrict__ sorted_idx,
+                                                          int32_t* __restrict__ row_map) {
+  // slot = round * 4 + wave, 16 slots of 64 consecutive flat indices each
+  extern __shared__ int h[];  // [16][E]
+  constexpr int kSlots = kChunk / 64;
+  for (int i = threadIdx.x; i < kSlots * E; i += 256) h[i] = 0;
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t base = (int64_t)blockIdx.x * kChunk;
+  int eid[kChunk / 256], rank[kChunk / 256];
+#pragma unroll
+  for (int it = 0; it < kChunk / 256; it++) {
+    const int e = load_id(ids, base + it * 256 + threadIdx.x, n, E);
+    // lanes of this wave holding the same expert id
+    unsigned long long peers = __ballot(e >= 0);
+    if (e < 0) peers = ~peers;
+    for (int b = 0; (1 << b) < E; b++) {
+      const unsigned long long vote = __ballot((e >> b) & 1);
+      peers &= ((e >> b) & 1) ? vote : ~vote;
+    }
+    const unsigned long long below = peers & ((1ull << lane) - 1ull);
+    eid[it] = e;
+    rank[it] = __popcll(below);
+    if (e >= 0 && below == 0) h[(it * 4 + wave) * E + e] = __popcll(peers);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int64_t run = goff[e] + hist[(int64_t)e * nchunk + blockIdx.x];
+    for (int sl = 0; sl < kSlots; sl++) {
+      const int c = h[sl * E + e];
+      h[sl * E + e] = (int)run;
+      run += c;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < kChunk / 256; it++) {
+    const int64_t flat = base + it * 256 + threadIdx.x;
+    if (flat >= n) continue;
+    if (eid[it] < 0) {
+      row_map[flat] = -1;
+      continue;
+    }
+    const int pos = h[(it * 4 + wave) * E + eid[it]] + rank[it];
+    row_map[flat] = pos;
+    if (sorted_idx) sorted_idx[pos] = flat;
+  }
+}
+
+}  // namespace aamd
+
+using namespace aamd;
+
+extern "C" int aamd_unpermute_combine(const void* y, int64_t M, int64_t H, const int32_t* row_map,
+                                      const void* probs, int probs_dtype, int64_t T, int topk, void* out,
+                                      void* stream) {
+  AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs_dtype == AAMD_BF16 || probs_dtype == AAMD_F32,
+               "unpermute_combine: unsupported probs dtype %d", probs_dtype);
+  AAMD_REQUIRE(M >= 0 && H >= 0 && T >= 0 && H % 8 == 0, "unpermute_combine: H=%lld must be a multiple of 8",
+               (long long)H);
+  AAMD_REQUIRE(topk >= 1 && topk <= kMaxTopk, "unpermute_combine: topk=%d out of range [1, %d]", topk, kMaxTopk);
+  AAMD_REQUIRE(M < 0x7fffffffLL && T < 0x7fffffffLL, "unpermute_combine: too many rows");
+  if (T == 0 || H == 0) return AAMD_OK;
+  AAMD_REQUIRE(row_map && out && (y || M == 0), "unpermute_combine: null pointer");
+  AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs != nullptr, "unpermute_combine: probs missing");
+  AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0, "unpermute_combine: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int H8 = (int)(H / 8);
+  dim3 grid((unsigned)T), block(256);
+  if (probs_dtype == AAMD_BF16)
+    unpermute_combine_kernel<AAMD_BF16><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+  else if (probs_dtype == AAMD_F32)
+    unpermute_combine_kernel<AAMD_F32><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+  else
+    unpermute_combine_kernel<AAMD_NONE><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+  AAMD_LAUNCH_CHECK("unpermute_combine");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_permute_rows(const void* x, int x_dtype, int64_t T, int64_t cols, const int32_t* row_map,
+                                 int topk, int64_t M_out, void* out, void* stream) {
+  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32, "permute_rows: unsupported dtype %d", x_dtype);
+  const int64_t row_bytes = cols * (x_dtype == AAMD_BF16 ? 2 : 4);
+  AAMD_REQUIRE(T >= 0 && cols >= 0 && row_bytes % 16 == 0, "permute_rows: row size must be a multiple of 16 bytes");
+  AAMD_REQUIRE(topk >= 1 && M_out >= 0 && T < 0x7fffffffLL, "permute_rows: bad topk / sizes");
+  if (T == 0 || cols == 0) return AAMD_OK;
+  AAMD_REQUIRE(x && out && row_map, "permute_rows: null pointer");
+  AAMD_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "permute_rows: pointers must be 16-byte aligned");
+  permute_rows_kernel<<<(unsigned)T, 256, 0, (hipStream_t)stream>>>((const v4i*)x, (int)(row_bytes / 16), row_map, topk,
+                                                                    M_out, (v4i*)out);
+  AAMD_LAUNCH_CHECK("permute_rows");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_invert_permutation(const int64_t* sorted_idx, int64_t n_perm, int64_t n_flat, int32_t* row_map,
+                                       void* stream) {
+  AAMD_REQUIRE(n_perm >= 0 && n_flat >= 0 && n_perm <= n_flat, "invert_permutation: bad sizes");
+  AAMD_REQUIRE(n_flat < 0x7fffffffLL, "invert_permutation: too many rows");
+  if (n_flat == 0) return AAMD_OK;
+  AAMD_REQUIRE(row_map && (sorted_idx || n_perm == 0), "invert_permutation: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  if (n_perm < n_flat) {
+    fill_i32_kernel<<<(unsigned)((n_flat + 255) / 256), 256, 0, st>>>(row_map, n_flat, -1);
+    AAMD_LAUNCH_CHECK("fill_i32");
+  }
+  if (n_perm > 0) {
+    invert_permutation_kernel<<<(unsigned)((n_perm + 255) / 256), 256, 0, st>>>(sorted_idx, n_perm, n_flat, row_map);
+    AAMD_LAUNCH_CHECK("invert_permutation");
+  }
+  return AAMD_OK;
+}
+
+extern "C" int64_t aamd_moe_preprocess_ws_ints(int64_t n, int E) {
+  if (n < 0 || E < 1) return 0;
+  const int64_t nchunk = (n + kChunk - 1) / kChunk;
+  return (int64_t)E * (nchunk > 0 ? nchunk : 1) + E;
+}
+
+extern "C" int aamd_moe_preprocess(const void* expert_ids, int ids_are_i64, int64_t n, int E, int64_t* sorted_idx,
+                                   int32_t* row_map, int64_t* group_offsets, int32_t* ws, void* stream) {
+  AAMD_REQUIRE(n >= 0 && n < 0x7fffffffLL, "moe_preprocess: n out of range");
+  AAMD_REQUIRE(E >= 1 && E <= 1024, "moe_preprocess: E=%d out of range [1, 1024]", E);
+  AAMD_REQUIRE(group_offsets && ws, "moe_preprocess: group_offsets / ws required");
+  AAMD_REQUIRE(n == 0 || (expert_ids && row_map), "moe_preprocess: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int nchunk = (int)((n + kChunk - 1) / kChunk);
+  const int nc = nchunk > 0 ? nchunk : 1;
+  int32_t* hist = ws;
+  int32_t* totals = ws + (int64_t)E * nc;
+  if (nchunk == 0) {
+    fill_i32_kernel<<<(unsigned)((E + 255) / 256), 256, 0, st>>>(hist, E, 0);
+    AAMD_LAUNCH_CHECK("fill_i32");
+  } else if (ids_are_i64) {
+    route_hist_kernel<int64_t><<<nchunk, 256, E * sizeof(int), st>>>((const int64_t*)expert_ids, n, E, nc, hist);
+  } else {
+    route_hist_kernel<int32_t><<<nchunk, 256, E * sizeof(int), st>>>((const int32_t*)expert_ids, n, E, nc, hist);
+  }
+  AAMD_LAUNCH_CHECK("route_hist");
+  route_rowscan_kernel<<<E, 256, 0, st>>>(hist, nc, totals);
+  AAMD_LAUNCH_CHECK("route_rowscan");
+  route_goff_kernel<<<1, 256, 0, st>>>(totals, E, group_offsets);
+  AAMD_LAUNCH_CHECK("route_goff");
+  if (nchunk > 0) {
+    const size_t sh = (size_t)(kChunk / 64) * E * sizeof(int);
+    if (ids_are_i64)
+      route_place_kernel<int64_t><<<nchunk, 256, sh, st>>>((const int64_t*)expert_ids, n, E, nc, hist, group_offsets, sorted_idx, row_map);
+    else
+      route_place_kernel<int32_t><<<nchunk, 256, sh, st>>>((const int32_t*)expert_ids, n, E, nc, hist, group_offsets, sorted_idx, row_map);
+    AAMD_LAUNCH_CHECK("route_place");
+  }
+  return AAMD_OK;
+}

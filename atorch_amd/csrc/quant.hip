@@ -1,0 +1,426 @@
+// Memory-bound quantisation kernels for gfx950: 1x128 tile quant (optionally with the token
+// permute fused in as a scatter), row-wise + transposed quant of ragged groups in one pass,
+// 128x128 block quant with the transposed copy, and dequant.
+//
+// All of them stream HBM with 128-bit accesses; amax reductions over a 128-element tile run
+// inside one 16-lane DPP row.  Scales and codes are part of a bit-exact contract, so every
+// division is the IEEE one (no reciprocal tricks).
+#include "common.hpp"
+
+namespace aamd {
+
+// ---------------------------------------------------------------------------------------
+// tile loaders: 8 consecutive elements per lane
+// ---------------------------------------------------------------------------------------
+template <typename IN>
+struct Raw8;
+template <>
+struct Raw8<BF16> {
+  v4i a;
+  __device__ __forceinline__ void load(const u16* p) { a = *reinterpret_cast<const v4i*>(p); }
+  __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v) const { unpack8(a, v); }
+};
+template <>
+struct Raw8<F32> {
+  v4i a, b;
+  __device__ __forceinline__ void load(const float* p) {
+    a = reinterpret_cast<const v4i*>(p)[0];
+    b = reinterpret_cast<const v4i*>(p)[1];
+  }
+  __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v) const {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[i] = __int_as_float(a[i]);
+      v[4 + i] = __int_as_float(b[i]);
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------------------
+// 1x128 quant, 16 lanes per tile, U tiles per lane group.  SCATTER: write each quantised
+// row to its topk destinations (row_map), reading it once.
+// ---------------------------------------------------------------------------------------
+template <typename IN, bool SCATTER, int U>
+__global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::elem* __restrict__ x, int64_t ldx,
+                                                          int nt, int64_t total_tiles,
+                                                          const int32_t* __restrict__ row_map, int topk,
+                                                          uint8_t* __restrict__ q, float* __restrict__ s,
+                                                          float eps) {
+  const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
+  const int64_t base = (int64_t)blockIdx.x * (16 * U);
+  const int64_t cols = (int64_t)nt * kTile;
+
+  Raw8<IN> raw[U];
+  int64_t row[U];
+  int tc[U];
+  bool valid[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    int64_t tile = base + u * 16 + grp;
+    valid[u] = tile < total_tiles;
+    if (!valid[u]) tile = total_tiles - 1;
+    row[u] = tile / nt;
+    tc[u] = (int)(tile - row[u] * nt);
+    raw[u].load(x + row[u] * ldx + (int64_t)tc[u] * kTile + l * 8);
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    float v[8];
+    raw[u].get(v);
+    const float sc = scale_from_amax(row16_max(amax8(v)), eps);
+    const v2i codes = quant8(v, sc);
+    if (!valid[u]) continue;
+    if constexpr (!SCATTER) {
+      *reinterpret_cast<v2i*>(q + row[u] * cols + (int64_t)tc[u] * kTile + l * 8) = codes;
+      if (l == 0) s[row[u] * nt + tc[u]] = sc;
+    } else {
+      for (int j = 0; j < topk; j++) {
+        const int64_t dst = row_map[row[u] * topk + j];
+        if (dst < 0) continue;
+        *reinterpret_cast<v2i*>(q + dst * cols + (int64_t)tc[u] * kTile + l * 8) = codes;
+        if (l == 0) s[dst * nt + tc[u]] = sc;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// 128x128 register tile shared by the dual (row + transposed) quant and the block quant:
+// 256 threads, thread (gr = tid/16, c = tid%16) holds rows gr*8 .. gr*8+7, columns c*8 .. c*8+7.
+// ---------------------------------------------------------------------------------------
+constexpr int kTLd = kTile + 16;  // LDS row stride (bytes) of the transposed code tile
+
+template <typename IN>
+__device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, int64_t ldx, int rows_valid,
+                                          float (&v)[8][8]) {
+  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+  Raw8<IN> raw[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int r = gr * 8 + i;
+    if (r < rows_valid)
+      raw[i].load(x + (int64_t)r * ldx + c * 8);
+    else
+      raw[i].zero();
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) raw[i].get(v[i]);
+}
+
+// codes of the 8x8 register block, transposed through LDS, written as rows of 128 bytes:
+// out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
+__device__ __forceinline__ void store_transposed(const float (&v)[8][8], const float* cs, uint8_t* tile_t,
+                                                 uint8_t* __restrict__ out, int64_t ld_out) {
+  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    float col[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) col[i] = v[i][j];
+    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cs[j]);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < 4; n++) {
+    const int idx = threadIdx.x + 256 * n;
+    const int r = idx >> 3, ch = idx & 7;
+    *reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16) =
+        *reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16);
+  }
+}
+
+template <typename IN>
+__global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
+    const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
+    const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
+    uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps) {
+  __shared__ float part[16][kTile];
+  __shared__ float cscale[kTile];
+  __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
+  __shared__ int slot;
+
+  const int kc = blockIdx.x, pt = blockIdx.y;
+  const int g = find_group(tile_off, E, pt, &slot);
+  if (g >= E) return;
+  const int64_t cols = (int64_t)nt * kTile;
+  const int64_t m0 = goff[g] + (int64_t)(pt - tile_off[g]) * kTile;
+  const int64_t left = goff[g + 1] - m0;
+  const int mvalid = left < kTile ? (int)left : kTile;
+  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+
+  float v[8][8];
+  load_tile<IN>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v);
+
+  // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
+  float cm[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) cm[j] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) cm[j] = fmaxf(cm[j], fabsf(v[i][j]));
+    if (q != nullptr) {
+      const float sc = scale_from_amax(row16_max(amax8(v[i])), eps);
+      const int r = gr * 8 + i;
+      const v2i codes = quant8(v[i], sc);
+      if (r < mvalid) {
+        *reinterpret_cast<v2i*>(q + (m0 + r) * cols + (int64_t)kc * kTile + c * 8) = codes;
+        if (c == 0) s[(m0 + r) * nt + kc] = sc;
+      }
+    }
+  }
+  // column amax over the 128 tokens of the tile
+#pragma unroll
+  for (int j = 0; j < 8; j++) part[gr][c * 8 + j] = cm[j];
+  __syncthreads();
+  if (threadIdx.x < kTile) {
+    float m = part[0][threadIdx.x];
+#pragma unroll
+    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][threadIdx.x]);
+    const float sc = scale_from_amax(m, eps);
+    cscale[threadIdx.x] = sc;
+    s_t[(int64_t)pt * cols + (int64_t)kc * kTile + threadIdx.x] = sc;
+  }
+  __syncthreads();
+  float cs[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) cs[j] = cscale[c * 8 + j];
+  store_transposed(v, cs, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
+}
+
+template <typename IN>
+__global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::elem* __restrict__ w,
+                                                            int64_t expert_stride, int64_t N, int64_t K,
+                                                            uint8_t* __restrict__ q, float* __restrict__ s,
+                                                            uint8_t* __restrict__ q_t, float* __restrict__ s_t,
+                                                            float eps) {
+  __shared__ float part[16];
+  __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
+  const int kb = blockIdx.x, nb = blockIdx.y, e = blockIdx.z;
+  const int nkb = (int)(K / kTile), nnb = (int)(N / kTile);
+  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+
+  float v[8][8];
+  load_tile<IN>(w + e * expert_stride + (int64_t)nb * kTile * K + (int64_t)kb * kTile, K, kTile, v);
+  float m = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) m = fmaxf(m, amax8(v[i]));
+  m = row16_max(m);
+  if (c == 0) part[gr] = m;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; i++) m = fmaxf(m, part[i]);
+  const float sc = scale_from_amax(m, eps);
+  if (threadIdx.x == 0) {
+    s[((int64_t)e * nnb + nb) * nkb + kb] = sc;
+    if (s_t != nullptr) s_t[((int64_t)e * nkb + kb) * nnb + nb] = sc;
+  }
+  uint8_t* qe = q + (int64_t)e * N * K + (int64_t)nb * kTile * K + (int64_t)kb * kTile;
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+    *reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8) = quant8(v[i], sc);
+  if (q_t != nullptr) {
+    float cs[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) cs[j] = sc;
+    store_transposed(v, cs, tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, N);
+  }
+}
+
+// tile_off[e] = sum_{j<e} ceil(rows_j / tile); one block, any E.
+__global__ __launch_bounds__(256) void group_tile_offsets_kernel(const int64_t* __restrict__ goff, int E, int tile,
+                                                                 int32_t* __restrict__ tile_off) {
+  __shared__ int buf[256];
+  __shared__ int carry;
+  if (threadIdx.x == 0) {
+    carry = 0;
+    tile_off[0] = 0;
+  }
+  __syncthreads();
+  for (int base = 0; base < E; base += 256) {
+    const int e = base + threadIdx.x;
+    int n = 0;
+    if (e < E) n = (int)((goff[e + 1] - goff[e] + tile - 1) / tile);
+    buf[threadIdx.x] = n;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+      __syncthreads();
+      buf[threadIdx.x] += t;
+      __syncthreads();
+    }
+    if (e < E) tile_off[e + 1] = carry + buf[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 255) carry += buf[255];
+    __syncthreads();
+  }
+}
+
+template <typename OUT>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ q, const float* __restrict__ s,
+                                                      int64_t M, int64_t N, int tile_scale,
+                                                      OUT* __restrict__ y) {
+  // one lane: 16 consecutive codes of one row
+  const int64_t chunks_per_row = N / 16;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * chunks_per_row) return;
+  const int64_t r = idx / chunks_per_row, ch = idx - r * chunks_per_row;
+  const int64_t nt = N / kTile;
+  const float sc = tile_scale ? s[r * nt + ch / 8] : s[(r / kTile) * nt + ch / 8];
+  const v4i raw = *reinterpret_cast<const v4i*>(q + r * N + ch * 16);
+  float o[16];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(raw[i], false);
+    auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(raw[i], true);
+    o[4 * i] = lo[0] * sc;
+    o[4 * i + 1] = lo[1] * sc;
+    o[4 * i + 2] = hi[0] * sc;
+    o[4 * i + 3] = hi[1] * sc;
+  }
+  OUT* dst = y + r * N + ch * 16;
+  if constexpr (sizeof(OUT) == 4) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      reinterpret_cast<v4f*>(dst)[i] = v4f{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+  } else {
+    v4i w0, w1;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      w0[i] = (int)(f32_to_bf16_bits(o[2 * i]) | (f32_to_bf16_bits(o[2 * i + 1]) << 16));
+      w1[i] = (int)(f32_to_bf16_bits(o[8 + 2 * i]) | (f32_to_bf16_bits(o[8 + 2 * i + 1]) << 16));
+    }
+    reinterpret_cast<v4i*>(dst)[0] = w0;
+    reinterpret_cast<v4i*>(dst)[1] = w1;
+  }
+}
+
+int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st) {
+  group_tile_offsets_kernel<<<1, 256, 0, st>>>(goff, E, tile, tile_off);
+  AAMD_LAUNCH_CHECK("group_tile_offsets");
+  return AAMD_OK;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace aamd
+
+using namespace aamd;
+
+extern "C" int aamd_quant_1x128(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ldx, uint8_t* q,
+                                float* s, float eps, void* stream) {
+  return aamd_permute_quant_1x128(x, x_dtype, rows, cols, ldx, nullptr, 1, rows, q, s, eps, stream);
+}
+
+extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
+                                        const int32_t* row_map, int topk, int64_t M_out, uint8_t* q, float* s,
+                                        float eps, void* stream) {
+  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32, "quant_1x128: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(T >= 0 && cols >= 0 && cols % kTile == 0, "quant_1x128: cols=%lld must be a multiple of 128",
+               (long long)cols);
+  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "quant_1x128: ldx=%lld must be >= cols and a multiple of 8",
+               (long long)ldx);
+  AAMD_REQUIRE(topk >= 1 && M_out >= 0, "quant_1x128: bad topk/M_out");
+  if (T == 0 || cols == 0) return AAMD_OK;
+  AAMD_REQUIRE(x && q && s, "quant_1x128: null pointer");
+  AAMD_REQUIRE(aligned16(x) && aligned16(q), "quant_1x128: x and q must be 16-byte aligned");
+  const int nt = (int)(cols / kTile);
+  const int64_t total = T * nt;
+  AAMD_REQUIRE(total < (int64_t)1 << 40, "quant_1x128: too many tiles");
+  hipStream_t st = (hipStream_t)stream;
+  constexpr int U = 4;
+  const int64_t blocks = (total + 16 * U - 1) / (16 * U);
+  AAMD_REQUIRE(blocks < 0x7fffffffLL, "quant_1x128: grid too large");
+  dim3 grid((unsigned)blocks), block(256);
+  if (row_map == nullptr) {
+    if (x_dtype == AAMD_BF16)
+      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, q, s, eps);
+    else
+      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, q, s, eps);
+  } else {
+    if (x_dtype == AAMD_BF16)
+      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, q, s, eps);
+    else
+      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, q, s, eps);
+  }
+  AAMD_LAUNCH_CHECK("quant_1x128");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t M, int64_t cols, int64_t ldx,
+                                             const int64_t* group_offsets, int E, int32_t* tile_ws, uint8_t* q,
+                                             float* s, uint8_t* q_t, float* s_t, int64_t ld_t, float eps,
+                                             void* stream) {
+  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32, "quant_dual: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(M >= 0 && cols >= 0 && cols % kTile == 0, "quant_dual: cols=%lld must be a multiple of 128",
+               (long long)cols);
+  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "quant_dual: bad ldx=%lld", (long long)ldx);
+  AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "quant_dual: group_offsets / tile_ws required");
+  AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
+  AAMD_REQUIRE((q == nullptr) == (s == nullptr), "quant_dual: q and s go together");
+  AAMD_REQUIRE(q_t && s_t, "quant_dual: q_t / s_t required");
+  if (cols == 0) return AAMD_OK;
+  // sum_g ceil(M_g/128) <= floor(M/128) + E; the caller's ld_t must hold the real total,
+  // which only the device knows: every tile beyond ld_t/128 would be out of bounds, so the
+  // grid is clamped to ld_t/128 padded tiles and ld_t is required to cover the upper bound
+  // whenever the bound is what the caller used.
+  const int64_t max_tiles = M / kTile + E;
+  const int64_t grid_tiles = ld_t / kTile < max_tiles ? ld_t / kTile : max_tiles;
+  if (grid_tiles == 0) return AAMD_OK;
+  AAMD_REQUIRE(aligned16(x) && aligned16(q_t) && (!q || aligned16(q)), "quant_dual: pointers must be 16-byte aligned");
+  AAMD_REQUIRE(grid_tiles <= 65535, "quant_dual: more than 65535 token tiles");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
+  if (rc) return rc;
+  dim3 grid((unsigned)(cols / kTile), (unsigned)grid_tiles), block(256);
+  const int nt = (int)(cols / kTile);
+  if (x_dtype == AAMD_BF16)
+    quant_dual_grouped_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+  else
+    quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+  AAMD_LAUNCH_CHECK("quant_dual_grouped");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_quant_128x128(const void* w, int w_dtype, int64_t E, int64_t N, int64_t K,
+                                  int64_t expert_stride, uint8_t* q, float* s, uint8_t* q_t, float* s_t, float eps,
+                                  void* stream) {
+  AAMD_REQUIRE(w_dtype == AAMD_BF16 || w_dtype == AAMD_F32, "quant_128x128: unsupported dtype %d", w_dtype);
+  AAMD_REQUIRE(E >= 0 && N >= 0 && K >= 0 && N % kTile == 0 && K % kTile == 0,
+               "quant_128x128: N=%lld and K=%lld must be multiples of 128", (long long)N, (long long)K);
+  AAMD_REQUIRE((q_t == nullptr) == (s_t == nullptr), "quant_128x128: q_t and s_t go together");
+  if (E == 0 || N == 0 || K == 0) return AAMD_OK;
+  AAMD_REQUIRE(w && q && s, "quant_128x128: null pointer");
+  AAMD_REQUIRE(expert_stride >= N * K && expert_stride % 8 == 0, "quant_128x128: bad expert stride");
+  AAMD_REQUIRE(aligned16(w) && aligned16(q) && (!q_t || aligned16(q_t)), "quant_128x128: pointers must be 16-byte aligned");
+  AAMD_REQUIRE(N / kTile <= 65535 && E <= 65535, "quant_128x128: grid too large");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)(K / kTile), (unsigned)(N / kTile), (unsigned)E), block(256);
+  if (w_dtype == AAMD_BF16)
+    quant_128x128_kernel<BF16><<<grid, block, 0, st>>>((const u16*)w, expert_stride, N, K, q, s, q_t, s_t, eps);
+  else
+    quant_128x128_kernel<F32><<<grid, block, 0, st>>>((const float*)w, expert_stride, N, K, q, s, q_t, s_t, eps);
+  AAMD_LAUNCH_CHECK("quant_128x128");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_dequant(const uint8_t* q, const float* s, int64_t M, int64_t N, int tile_scale, void* y,
+                            int y_dtype, void* stream) {
+  AAMD_REQUIRE(y_dtype == AAMD_BF16 || y_dtype == AAMD_F32, "dequant: unsupported dtype %d", y_dtype);
+  AAMD_REQUIRE(M >= 0 && N >= 0 && N % kTile == 0, "dequant: N=%lld must be a multiple of 128", (long long)N);
+  AAMD_REQUIRE(tile_scale || M % kTile == 0, "dequant: block scales need M %% 128 == 0");
+  if (M == 0 || N == 0) return AAMD_OK;
+  AAMD_REQUIRE(q && s && y && aligned16(q) && aligned16(y), "dequant: null or unaligned pointer");
+  const int64_t n = M * (N / 16);
+  const int64_t blocks = (n + 255) / 256;
+  AAMD_REQUIRE(blocks < 0x7fffffffLL, "dequant: grid too large");
+  hipStream_t st = (hipStream_t)stream;
+  if (y_dtype == AAMD_F32)
+    dequant_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(q, s, M, N, tile_scale, (float*)y);
+  else
+    dequant_kernel<u16><<<(unsigned)blocks, 256, 0, st>>>(q, s, M, N, tile_scale, (u16*)y);
+  AAMD_LAUNCH_CHECK("dequant");
+  return AAMD_OK;
+}

@@ -1,0 +1,184 @@
+/*
+ * C ABI of libatorch_amd_fp8.so: hand-written gfx950 (MI355X) kernels for the
+ * FP8 grouped-linear MoE expert path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller (the caller
+ *     allocates all outputs and workspaces); nothing here allocates device
+ *     memory or synchronises the host with the device;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     kernels are only enqueued;
+ *   - functions return AAMD_OK (0) or an error code; aamd_last_error() gives
+ *     the message of the last failure on the calling thread;
+ *   - fp8 tensors are OCP e4m3fn codes, one byte each; scales are fp32
+ *     dequantisation scales  s = max(amax, eps) / 448  (0 -> 1);
+ *   - `dtype` arguments: AAMD_BF16 or AAMD_F32 (also AAMD_NONE where stated).
+ *
+ * Each entry point names the reference interface it replaces (paths relative
+ * to the reference tree root).
+ */
+#ifndef ATORCH_AMD_FP8_H
+#define ATORCH_AMD_FP8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AAMD_OK 0
+#define AAMD_ERR_ARG 1 /* bad shape / alignment / dtype */
+#define AAMD_ERR_HIP 2 /* the HIP runtime refused the launch */
+
+#define AAMD_NONE (-1)
+#define AAMD_BF16 0
+#define AAMD_F32 1
+
+#define AAMD_ABI_VERSION 1
+
+/* Library identity and error text. */
+int aamd_abi_version(void);
+const char *aamd_last_error(void);
+
+/*
+ * 1x128 tile quantisation.
+ * Replaces tile_quant / tile_quant_kernel, atorch/modules/fp8/triton_kernel.py:94-140
+ * (dispatch: Fp8Quantization.quantize_tilewise, atorch/modules/fp8/quantize.py:176-201).
+ *   x [rows, cols] (row stride ldx elements), cols % 128 == 0
+ *   q [rows, cols] codes, s [rows, cols/128] fp32, both dense.
+ */
+int aamd_quant_1x128(const void *x, int x_dtype, int64_t rows, int64_t cols, int64_t ldx, uint8_t *q, float *s,
+                     float eps, void *stream);
+
+/*
+ * Token permute fused into the 1x128 quantisation: every token row is read and
+ * quantised once and written to its topk destination rows.
+ * Replaces permute (atorch/modules/moe/token_dispatcher.py:89-116) followed by the
+ * per-expert quantize calls of atorch/modules/fp8/quantized_grouped_linear.py:90-101.
+ *   x [T, cols]; row_map [T*topk] int32: destination (permuted) row of flat
+ *   index token*topk+slot, or -1 when that copy is dropped;
+ *   q [M_out, cols], s [M_out, cols/128] dense; rows no map entry points to are not written.
+ */
+int aamd_permute_quant_1x128(const void *x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
+                             const int32_t *row_map, int topk, int64_t M_out, uint8_t *q, float *s, float eps,
+                             void *stream);
+
+/*
+ * Token permute without quantisation (rows of bf16 or fp32 copied to their topk permuted
+ * positions, each source row read once).
+ * Replaces permute, atorch/modules/moe/token_dispatcher.py:89-116 (index_select on the argsort).
+ *   x [T, cols] dense; out [M_out, cols] dense; cols * element size must be a multiple of 16.
+ */
+int aamd_permute_rows(const void *x, int x_dtype, int64_t T, int64_t cols, const int32_t *row_map, int topk,
+                      int64_t M_out, void *out, void *stream);
+
+/*
+ * Row-wise AND transposed 1x128 quantisation of ragged groups in one pass over x
+ * ("return_transpose=True").
+ * Replaces quantize_op.quantize(x_i, params, return_transpose=True) per expert,
+ * quantized_grouped_linear.py:90-101 and :200-206; the transposed result is defined
+ * in-tree as tile_quant(x_i.t().contiguous()), atorch/modules/fp8/scaled_linear.py:402-414,
+ * with a partial last token tile zero padded.
+ *   x [M, cols]; group_offsets [E+1] int64 (device) exclusive prefix of rows per group;
+ *   q [M, cols], s [M, cols/128]              (both may be NULL: transposed only)
+ *   q_t [cols, ld_t]: q_t[c, poff_g + m] = code of x[off_g + m, c], where
+ *       poff_g = sum_{j<g} ceil(M_j/128)*128; pad columns of a group are written 0
+ *   s_t [ld_t/128, cols]: s_t[poff_g/128 + m/128, c]
+ *   ld_t % 128 == 0 and ld_t >= poff_E (M + 127*E rounded up to 128 always suffices)
+ *   tile_ws: E+1 int32 of scratch.
+ */
+int aamd_quant_1x128_dual_grouped(const void *x, int x_dtype, int64_t M, int64_t cols, int64_t ldx,
+                                  const int64_t *group_offsets, int E, int32_t *tile_ws, uint8_t *q, float *s,
+                                  uint8_t *q_t, float *s_t, int64_t ld_t, float eps, void *stream);
+
+/*
+ * 128x128 block quantisation of E weight matrices, optionally also emitting the
+ * transposed codes and scale grid.
+ * Replaces block_quant / block_quant_kernel, triton_kernel.py:21-46 (dispatch
+ * quantize.py:204-232) and w_fp8.t().contiguous() / scale.t().contiguous(),
+ * scaled_linear.py:359-365.
+ *   w [E, N, K] (expert stride in elements; rows dense), N % 128 == 0, K % 128 == 0
+ *   q [E, N, K], s [E, N/128, K/128]; q_t [E, K, N], s_t [E, K/128, N/128] (q_t/s_t may be NULL).
+ */
+int aamd_quant_128x128(const void *w, int w_dtype, int64_t E, int64_t N, int64_t K, int64_t expert_stride,
+                       uint8_t *q, float *s, uint8_t *q_t, float *s_t, float eps, void *stream);
+
+/*
+ * Dequantisation y = code * scale.
+ * Replaces dequant, triton_kernel.py:49-91.  tile_scale != 0: s [M, N/128]; else s [M/128, N/128].
+ */
+int aamd_dequant(const uint8_t *q, const float *s, int64_t M, int64_t N, int tile_scale, void *y, int y_dtype,
+                 void *stream);
+
+/*
+ * Ragged grouped block-scaled GEMM, "NT": for every group g and its rows m,
+ *   C[m, n] = sum_kb dot(A[m, kb], B_g[n, kb]) * a_s[m, kb] * b_s_g[n/128 or n, kb]  (+ bias_g[n])
+ * fp8 x fp8 MFMA, fp32 accumulation, scales applied per 128-deep block.
+ * Replaces fp8_gemm / fp8_gemm_kernel, triton_kernel.py:143-210, and
+ * quantize_op.grouped_qgemm for fprop and dgrad, quantized_grouped_linear.py:141-151, 214-223.
+ *   a [M, K] codes (row stride lda bytes), a_s [M, K/128]
+ *   b [E, N, K] codes dense, b_s [E, N/128, K/128] (b_tile_scaled == 0) or [E, N, K/128] (!= 0)
+ *   group_offsets [E+1] int64 device, or NULL for a single group [0, M] (then E must be 1)
+ *   c [M, N] of c_dtype (row stride ldc elements); rows of empty groups are not touched
+ *   bias [E, N] of bias_dtype or NULL (AAMD_NONE); tile_ws: E+1 int32 scratch.
+ *   K % 128 == 0, N % 128 == 0.
+ */
+int aamd_grouped_gemm_fp8_nt(const uint8_t *a, int64_t lda, const float *a_s, const uint8_t *b, const float *b_s,
+                             int b_tile_scaled, const int64_t *group_offsets, int E, int32_t *tile_ws, int64_t M,
+                             int64_t N, int64_t K, void *c, int c_dtype, int64_t ldc, const void *bias,
+                             int bias_dtype, void *stream);
+
+/*
+ * Grouped weight-gradient GEMM: dW_g[n, k] (+)= sum over the tokens m of group g of
+ * dY[m, n] * X[m, k], both operands 1x128-scaled along the tokens (layouts of
+ * aamd_quant_1x128_dual_grouped's q_t / s_t).
+ * Replaces quantize_op.grouped_qgemm(qdy_t, qx_t, mm_wgrad, ..., accumulate=...),
+ * quantized_grouped_linear.py:243-253.
+ *   dyt [N, ld_t], sdyt [ld_t/128, N]; xt [K, ld_t], sxt [ld_t/128, K]
+ *   dw [E, N, K] of dw_dtype (expert stride in elements); an empty group gives zeros,
+ *   or leaves dw_g untouched when accumulate != 0.
+ */
+int aamd_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uint8_t *xt, const float *sxt,
+                                int64_t ld_t, const int64_t *group_offsets, int E, int32_t *tile_ws, int64_t N,
+                                int64_t K, void *dw, int dw_dtype, int64_t expert_stride, int accumulate,
+                                void *stream);
+
+/*
+ * Inverse permutation + weighted combine in one gather-reduce pass:
+ *   out[t, :] = sum_j probs[t, j] * y[row_map[t*topk + j], :]
+ * Replaces unpermute, token_dispatcher.py:119-161 (zeros + index_copy_ + multiply + sum).
+ * Each product is rounded to the promoted dtype before the fp32 sum, as the reference's
+ * separate multiply and sum do (:156-159).
+ *   y [M, H] bf16; row_map [T*topk] int32 (-1 = dropped copy, contributes 0)
+ *   probs [T, topk] of probs_dtype (AAMD_BF16 -> out bf16; AAMD_F32 -> out fp32;
+ *   AAMD_NONE -> probs ignored, out bf16); H % 8 == 0.
+ */
+int aamd_unpermute_combine(const void *y, int64_t M, int64_t H, const int32_t *row_map, const void *probs,
+                           int probs_dtype, int64_t T, int topk, void *out, void *stream);
+
+/*
+ * Router preprocess on the device, no host round trip: histogram of expert ids,
+ * exclusive scan, stable counting sort.
+ * Replaces the argsort of permute (token_dispatcher.py:107-112) and the histc + .cpu()
+ * of MoEAllToAllTokenDispatcher.preprocess (token_dispatcher.py:297-353).
+ *   expert_ids [n] (n = T*topk; int64 when ids_are_i64 != 0, else int32), values in [0, E)
+ *   sorted_idx [n] int64: flat index of permuted row j (the reference's sorted_indices); may be NULL
+ *   row_map [n] int32: permuted row of flat index i (inverse of sorted_idx)
+ *   group_offsets [E+1] int64: exclusive prefix of tokens per expert
+ *   ws: aamd_moe_preprocess_ws_ints(n, E) int32 of scratch.
+ */
+int64_t aamd_moe_preprocess_ws_ints(int64_t n, int E);
+int aamd_moe_preprocess(const void *expert_ids, int ids_are_i64, int64_t n, int E, int64_t *sorted_idx,
+                        int32_t *row_map, int64_t *group_offsets, int32_t *ws, void *stream);
+
+/*
+ * row_map[sorted_idx[j]] = j for j < n_perm, -1 elsewhere (n_flat entries).
+ * Adapter from the reference's sorted_indices (token_dispatcher.py:112,136) to row_map.
+ */
+int aamd_invert_permutation(const int64_t *sorted_idx, int64_t n_perm, int64_t n_flat, int32_t *row_map,
+                            void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ATORCH_AMD_FP8_H */

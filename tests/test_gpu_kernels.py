@@ -1,0 +1,342 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle, at sizes the oracle
+finishes in seconds.  Bit-exact for codes, scales and index work; GEMM outputs within
+max relative error 1e-2 (bf16 out, fp32 accumulate)."""
+import pytest
+import torch
+
+from helpers import TILE, heavy_tailed, ragged_splits, randn_bf16, rel_err, topk_routing
+
+pytestmark = pytest.mark.gpu
+
+GEMM_TOL = 1e-2
+
+
+def _u8(t):
+    return t.view(torch.uint8).cpu()
+
+
+# ------------------------------------------------------------------------------------------
+# a1: 1x128 quant
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 128), (7, 256), (2048, 512), (33, 7168)])
+def test_tile_quant_matches_oracle(oracle, dev, dtype, shape):
+    from atorch_amd import kernels
+
+    x = heavy_tailed(shape, seed=shape[0], dtype=dtype)
+    q, s = kernels.tile_quant(x.to(dev))
+    qo, so = oracle.tile_quant(x)
+    assert torch.equal(s.cpu(), so)
+    assert torch.equal(_u8(q), qo)
+
+
+def test_tile_quant_all_bf16_patterns(oracle, dev):
+    """Every bf16 bit pattern as an element, for several tile maxima: pins the division and the
+    hardware fp8 conversion (RNE, subnormals) against the integer encoder of the oracle."""
+    from atorch_amd import kernels
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = bits[torch.isfinite(bits.float())]
+    rows = []
+    for amax in (1.0, 448.0, 3.0e-3, 1.7e4, 2.0**-120, 6.0e37, 1.0e-38):
+        v = finite[finite.float().abs() <= amax]
+        pad = (-v.numel()) % (TILE - 1)
+        v = torch.cat([v, torch.zeros(pad, dtype=torch.bfloat16)])
+        v = v.view(-1, TILE - 1)
+        col = torch.full((v.shape[0], 1), amax, dtype=torch.bfloat16)
+        rows.append(torch.cat([col, v], dim=1))
+    x = torch.cat(rows).contiguous()
+    q, s = kernels.tile_quant(x.to(dev))
+    qo, so = oracle.tile_quant(x)
+    assert torch.equal(s.cpu(), so)
+    assert torch.equal(_u8(q), qo)
+
+
+def test_tile_quant_known_answers(dev):
+    """zeros -> s = 1, codes 0; ones -> s = fl(1/448), codes 0x7E; rows of 1000 / -512 -> +-448
+    (atorch/tests/common_tests/scaled_linear_test.py:131-133, 305-311)."""
+    from atorch_amd import kernels
+
+    x = torch.ones(4, 256, dtype=torch.bfloat16)
+    x[0] = 0
+    x[1] = 1000
+    x[2] = -512
+    q, s = kernels.tile_quant(x.to(dev))
+    q, s = _u8(q), s.cpu()
+    assert torch.all(s[0] == 1.0) and torch.all(q[0] == 0)
+    assert torch.all(s[1] == torch.tensor(1000.0) / 448.0) and torch.all(q[1] == 0x7E)
+    assert torch.all(s[2] == torch.tensor(512.0) / 448.0) and torch.all(q[2] == 0xFE)
+    assert torch.all(s[3] == torch.tensor(1.0) / 448.0) and torch.all(q[3] == 0x7E)
+
+
+def test_tile_quant_eps(oracle, dev):
+    from atorch_amd import kernels
+
+    x = randn_bf16((16, 256), 3, std=1e-3)
+    q, s = kernels.tile_quant(x.to(dev), eps=0.5)
+    qo, so = oracle.tile_quant(x, eps=0.5)
+    assert torch.equal(s.cpu(), so) and torch.equal(_u8(q), qo)
+
+
+def test_tile_quant_rejects_bad_shapes(dev):
+    from atorch_amd import kernels
+
+    with pytest.raises(AssertionError):
+        kernels.tile_quant(torch.zeros(4, 100, dtype=torch.bfloat16, device=dev))
+
+
+# ------------------------------------------------------------------------------------------
+# a1 + a9: permute fused into the quant; a9 alone; a11 preprocess
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,E,k", [(64, 4, 1), (1000, 8, 2), (777, 64, 8), (3000, 200, 4)])
+def test_moe_preprocess_matches_stable_sort(oracle, dev, T, E, k):
+    from atorch_amd import kernels
+
+    idx, _ = topk_routing(T, E, k, seed=T, zipf_s=1.2 if E >= 64 else None)
+    sorted_idx, row_map, goff = kernels.moe_preprocess(idx.to(dev), E)
+    so, counts = oracle.permute_indices(idx, E)
+    assert torch.equal(sorted_idx.cpu(), so)
+    assert torch.equal(sorted_idx.cpu(), torch.argsort(idx.reshape(-1), stable=True))
+    assert torch.equal(goff.cpu()[1:] - goff.cpu()[:-1], counts)
+    inv = torch.empty(T * k, dtype=torch.int32)
+    inv[so] = torch.arange(T * k, dtype=torch.int32)
+    assert torch.equal(row_map.cpu(), inv)
+
+
+def test_moe_preprocess_int32_ids_and_empty(dev):
+    from atorch_amd import kernels
+
+    idx = torch.tensor([3, 3, 0, 3], dtype=torch.int32)
+    sorted_idx, row_map, goff = kernels.moe_preprocess(idx.to(dev), 5)
+    assert sorted_idx.cpu().tolist() == [2, 0, 1, 3]
+    assert goff.cpu().tolist() == [0, 1, 1, 1, 4, 4]
+    s2, r2, g2 = kernels.moe_preprocess(torch.zeros(0, dtype=torch.int64, device=dev), 3)
+    assert s2.numel() == 0 and g2.cpu().tolist() == [0, 0, 0, 0]
+
+
+@pytest.mark.parametrize("T,E,k,H", [(512, 8, 2, 512), (300, 64, 8, 1024)])
+def test_permute_quant_commutes(oracle, dev, T, E, k, H):
+    """quant is row local, so permute(quant(x)) == quant(permute(x)) on codes and scales."""
+    from atorch_amd import kernels
+
+    x = heavy_tailed((T, H), seed=11)
+    idx, _ = topk_routing(T, E, k, seed=5)
+    sorted_idx, row_map, goff = kernels.moe_preprocess(idx.to(dev), E)
+    q, s = kernels.permute_tile_quant(x.to(dev), row_map, k, T * k)
+    xp, so, _ = oracle.permute(x, idx, E)
+    qo, sco = oracle.tile_quant(xp)
+    assert torch.equal(_u8(q), qo) and torch.equal(s.cpu(), sco)
+    # the un-quantised permute and the reference-shaped functions
+    from atorch_amd.token_dispatcher import permute
+
+    p, si = permute(x.to(dev), idx.to(dev), num_experts=E)
+    assert torch.equal(p.cpu(), xp) and torch.equal(si.cpu(), so)
+    p2, si2 = permute(x.to(dev), idx.to(dev))
+    assert torch.equal(p2.cpu(), xp) and torch.equal(si2.cpu(), so)
+
+
+# ------------------------------------------------------------------------------------------
+# a10: unpermute + combine
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("probs_dtype", [torch.bfloat16, torch.float32, None])
+@pytest.mark.parametrize("T,E,k,H", [(256, 8, 2, 512), (100, 64, 8, 1024)])
+def test_unpermute_combine(oracle, dev, probs_dtype, T, E, k, H):
+    from atorch_amd.token_dispatcher import unpermute
+
+    if probs_dtype is None:
+        k = 1
+    idx, probs = topk_routing(T, E, k, seed=9)
+    so, _ = oracle.permute_indices(idx, E)
+    y = randn_bf16((T * k, H), 21)
+    pr = None if probs_dtype is None else probs.to(probs_dtype)
+    out = unpermute(y.to(dev), so.to(dev), None if pr is None else pr.to(dev))
+    ref = oracle.unpermute(y, so, pr)
+    assert out.dtype == ref.dtype
+    assert torch.equal(out.cpu(), ref)
+    # against the torch restatement of the reference: <= 1 ulp of the output type
+    tref = oracle.torch_unpermute(y, so, pr)
+    assert tref.dtype == ref.dtype
+    torch.testing.assert_close(out.cpu().float(), tref.float(), rtol=2**-7 if ref.dtype == torch.bfloat16 else 1e-6, atol=1e-6)
+
+
+def test_unpermute_inverts_permute_top1(dev):
+    from atorch_amd.token_dispatcher import permute, unpermute
+
+    x = randn_bf16((333, 256), 2).to(dev)
+    idx = torch.randint(0, 7, (333,), generator=torch.Generator().manual_seed(0)).to(dev)
+    p, si = permute(x, idx, num_experts=7)
+    assert torch.equal(unpermute(p, si), x)
+
+
+# ------------------------------------------------------------------------------------------
+# a2 + a4: block quant
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("E,N,K", [(1, 128, 128), (3, 256, 384), (4, 1024, 512)])
+def test_block_quant_matches_oracle(oracle, dev, dtype, E, N, K):
+    from atorch_amd import kernels
+
+    w = randn_bf16((E, N, K), seed=N + K, std=0.02, dtype=dtype)
+    w[0, :128, :128] = 0  # an all-zero block -> scale 1
+    q, s, q_t, s_t = kernels.block_quant_batched(w.to(dev), return_transpose=True)
+    for e in range(E):
+        qo, so = oracle.block_quant(w[e])
+        assert torch.equal(s[e].cpu(), so) and torch.equal(_u8(q[e]), qo)
+        assert torch.equal(_u8(q_t[e]), qo.t()) and torch.equal(s_t[e].cpu(), so.t())
+    assert s[0, 0, 0].item() == 1.0
+    q1, s1 = kernels.block_quant(w[0].to(dev))
+    assert torch.equal(_u8(q1), _u8(q[0])) and torch.equal(s1.cpu(), s[0].cpu())
+
+
+# ------------------------------------------------------------------------------------------
+# a3: row-wise + transposed quant of ragged groups
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,K,E,mult", [(512, 256, 4, 128), (1000, 384, 6, 16), (777, 128, 5, 1)])
+def test_dual_grouped_quant(oracle, dev, dtype, M, K, E, mult):
+    from atorch_amd import kernels
+
+    x = heavy_tailed((M, K), seed=M, dtype=dtype)
+    splits = ragged_splits(M, E, seed=K, multiple=mult)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    q, s, q_t, s_t = kernels.tile_quant_dual_grouped(x.to(dev), goff, E)
+    qo, so = oracle.tile_quant(x)
+    assert torch.equal(_u8(q), qo) and torch.equal(s.cpu(), so)
+    qto, sto = oracle.tile_quant_t_grouped(x, splits, ld_t=q_t.shape[1])
+    ptot = oracle.padded_offsets(splits)[-1]
+    assert torch.equal(_u8(q_t)[:, :ptot], qto[:, :ptot])
+    assert torch.equal(s_t.cpu()[: ptot // TILE], sto[: ptot // TILE])
+    # transposed only
+    _, _, q_t2, s_t2 = kernels.tile_quant_dual_grouped(x.to(dev), goff, E, rowwise=False)
+    assert torch.equal(_u8(q_t2)[:, :ptot], qto[:, :ptot])
+
+
+def test_tile_quant_return_transpose_equals_quant_of_transpose(oracle, dev):
+    """M % 128 == 0: the transposed result is tile_quant(x.t().contiguous())
+    (atorch/modules/fp8/scaled_linear.py:404-414)."""
+    from atorch_amd import kernels
+
+    x = randn_bf16((256, 384), 4)
+    y, s, y_t, s_t = kernels.tile_quant(x.to(dev), return_transpose=True)
+    qo, so = oracle.tile_quant(x.t().contiguous())
+    assert y_t.shape == (384, 256) and s_t.shape == (384, 2)
+    assert torch.equal(_u8(y_t.contiguous()), qo) and torch.equal(s_t.cpu(), so)
+
+
+# ------------------------------------------------------------------------------------------
+# dequant
+# ------------------------------------------------------------------------------------------
+def test_dequant(oracle, dev):
+    from atorch_amd import kernels
+
+    x = randn_bf16((256, 384), 8)
+    q, s = kernels.tile_quant(x.to(dev))
+    d = kernels.dequant(q, s)
+    assert torch.equal(d.cpu(), oracle.dequant(_u8(q), s.cpu()))
+    qb, sb = kernels.block_quant(x.to(dev))
+    db = kernels.dequant(qb, sb, dtype=torch.bfloat16)
+    assert torch.equal(db.cpu(), oracle.dequant(_u8(qb), sb.cpu()).bfloat16())
+    # tile error <= block error (scaled_linear_test.py:305-319)
+    t = torch.ones(512, 512, dtype=torch.bfloat16)
+    t[1] = 1000
+    t[2] = -512
+    tq, ts = kernels.tile_quant(t.to(dev))
+    bq, bs = kernels.block_quant(t.to(dev))
+    et = (t.float() - kernels.dequant(tq, ts).cpu()).abs()
+    eb = (t.float() - kernels.dequant(bq, bs).cpu()).abs()
+    assert torch.all(eb >= et)
+
+
+# ------------------------------------------------------------------------------------------
+# a5/a6/a7: GEMMs
+# ------------------------------------------------------------------------------------------
+def _quant_inputs(oracle, M, N, K, E, seed):
+    x = randn_bf16((M, K), seed)
+    w = randn_bf16((E, N, K), seed + 1, std=0.02)
+    qx, sx = oracle.tile_quant(x)
+    qw = torch.stack([oracle.block_quant(w[e])[0] for e in range(E)])
+    sw = torch.stack([oracle.block_quant(w[e])[1] for e in range(E)])
+    return x, w, qx, sx, qw, sw
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (200, 256, 384), (64, 128, 1024), (513, 384, 256)])
+def test_fp8_gemm_dense(oracle, dev, M, N, K):
+    from atorch_amd import kernels
+
+    _, _, qx, sx, qw, sw = _quant_inputs(oracle, M, N, K, 1, seed=M + N)
+    ref = oracle.fp8_gemm(qx, sx, qw[0], sw[0])
+    for dt in (torch.bfloat16, torch.float32):
+        c = kernels.fp8_gemm(qx.to(dev).view(kernels.FP8), sx.to(dev), qw[0].to(dev).view(kernels.FP8), sw[0].to(dev), dtype=dt)
+        assert c.dtype == dt
+        assert rel_err(c.cpu(), ref) <= (GEMM_TOL if dt == torch.bfloat16 else 1e-5)
+    # textbook check: dequantise and multiply in fp64
+    full = (oracle.torch_dequant_tile(qx, sx).double() @ oracle.torch_dequant_block(qw[0], sw[0]).double().t())
+    assert rel_err(c.cpu(), full.float()) <= 1e-5
+
+
+def test_fp8_gemm_tile_scaled_b(oracle, dev):
+    from atorch_amd import kernels
+
+    M, N, K = 192, 256, 384
+    a, b = randn_bf16((M, K), 1), randn_bf16((N, K), 2)
+    qa, sa = oracle.tile_quant(a)
+    qb, sb = oracle.tile_quant(b)
+    ref = oracle.fp8_gemm(qa, sa, qb, sb)
+    c = kernels.fp8_gemm(qa.to(dev).view(kernels.FP8), sa.to(dev), qb.to(dev).view(kernels.FP8), sb.to(dev), dtype=torch.float32)
+    assert rel_err(c.cpu(), ref) <= 1e-5
+
+
+@pytest.mark.parametrize("M,N,K,E,mult", [(512, 256, 256, 4, 16), (1000, 128, 384, 6, 1), (300, 384, 128, 3, 128)])
+def test_grouped_gemm_nt(oracle, dev, M, N, K, E, mult):
+    from atorch_amd import kernels
+
+    _, _, qx, sx, qw, sw = _quant_inputs(oracle, M, N, K, E, seed=M)
+    splits = ragged_splits(M, E, seed=N, multiple=mult)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    ref = oracle.grouped_gemm_nt(qx, sx, qw, sw, splits)
+    bias = randn_bf16((E, N), 77)
+    args = (qx.to(dev).view(kernels.FP8), sx.to(dev), qw.to(dev).view(kernels.FP8), sw.to(dev), goff)
+    c32 = kernels.grouped_gemm_nt(*args, out_dtype=torch.float32)
+    assert rel_err(c32.cpu(), ref) <= 1e-5
+    c16 = kernels.grouped_gemm_nt(*args, out_dtype=torch.bfloat16)
+    assert rel_err(c16.cpu(), ref) <= GEMM_TOL
+    cb = kernels.grouped_gemm_nt(*args, out_dtype=torch.float32, bias=bias.to(dev))
+    refb = ref + torch.repeat_interleave(bias.float(), torch.tensor(splits), dim=0)
+    assert rel_err(cb.cpu(), refb) <= 1e-5
+    # grouped == per-expert loop, bit-wise (test_quantized_grouped_linear.py:735-737)
+    off = 0
+    for e, m in enumerate(splits):
+        if m:
+            ce = kernels.fp8_gemm(args[0][off : off + m].contiguous(), args[1][off : off + m].contiguous(), args[2][e], args[3][e], dtype=torch.bfloat16)
+            assert torch.equal(ce, c16[off : off + m])
+        off += m
+
+
+@pytest.mark.parametrize("M,N,K,E,mult", [(512, 128, 256, 4, 128), (1000, 256, 128, 6, 16), (333, 128, 128, 3, 1)])
+def test_grouped_gemm_wgrad(oracle, dev, M, N, K, E, mult):
+    from atorch_amd import kernels
+
+    x = randn_bf16((M, K), 1)
+    dy = randn_bf16((M, N), 2, std=1e-2)
+    splits = ragged_splits(M, E, seed=M, multiple=mult)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    ld_t = kernels.padded_total(splits)
+    qxt, sxt = oracle.tile_quant_t_grouped(x, splits, ld_t=ld_t)
+    qdt, sdt = oracle.tile_quant_t_grouped(dy, splits, ld_t=ld_t)
+    ref = oracle.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, splits)
+    args = (qdt.to(dev).view(kernels.FP8), sdt.to(dev), qxt.to(dev).view(kernels.FP8), sxt.to(dev), goff)
+    dw = kernels.grouped_gemm_wgrad(*args, out_dtype=torch.float32)
+    assert rel_err(dw.cpu(), ref) <= 1e-5
+    for e, m in enumerate(splits):
+        if m == 0:
+            assert torch.all(dw[e] == 0)
+    dw16 = kernels.grouped_gemm_wgrad(*args, out_dtype=torch.bfloat16)
+    assert rel_err(dw16.cpu(), ref) <= GEMM_TOL
+    # accumulate: second call adds; empty groups stay untouched
+    base = torch.rand(E, N, K, generator=torch.Generator().manual_seed(5))
+    acc = base.clone().to(dev)
+    kernels.grouped_gemm_wgrad(*args, out=acc, accumulate=True)
+    torch.testing.assert_close(acc.cpu(), base + ref, rtol=1e-5, atol=1e-6)
+    for e, m in enumerate(splits):
+        if m == 0:
+            assert torch.equal(acc[e].cpu(), base[e])
