@@ -50,6 +50,7 @@ struct GemmParams {
   int E;
   int nRt;         // Rrows / 128
   int nLt;         // kRaggedK: Lrows / 128
+  int max_kb;      // kRaggedK: contraction blocks the operand buffers hold (ld_t / 128)
   int accumulate;
   int bias_dtype;
 };
@@ -142,6 +143,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(const GemmParams p
     lvalid = kBM;
     kb0 = p.tile_off[g];
     nkb = p.tile_off[g + 1] - kb0;
+    if (kb0 + nkb > p.max_kb) nkb = p.max_kb > kb0 ? p.max_kb - kb0 : 0;  // never read past the buffers
   }
   g = __builtin_amdgcn_readfirstlane(g);
   const int64_t r0 = (int64_t)rt * kBN;
@@ -367,6 +369,7 @@ extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt
   p.bias = nullptr; p.bias_dtype = AAMD_NONE; p.bias_group_stride = 0;
   p.goff = group_offsets; p.tile_off = tile_ws;
   p.Lrows = N; p.Rrows = K; p.nkb = 0; p.E = E; p.nRt = (int)(K / kBN); p.nLt = (int)(N / kBM);
+  p.max_kb = (int)(ld_t / kBK);
   p.accumulate = accumulate;
   const int64_t blocks = (int64_t)E * p.nLt * p.nRt;
   return launch_gemm<kRaggedK, true>(p, dw_dtype, blocks, st);

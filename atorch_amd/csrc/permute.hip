@@ -2,6 +2,9 @@
 // counting sort), inverse permutation, and the fused unpermute + weighted combine.
 #include "common.hpp"
 
+// The combine reproduces "multiply, round, then sum": no fused multiply-add in this file.
+#pragma clang fp contract(off)
+
 namespace aamd {
 
 // ---------------------------------------------------------------------------------------
@@ -44,9 +47,10 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         float prod = v[i];
-        if constexpr (PD == AAMD_BF16) prod = bf16_bits_to_f32(f32_to_bf16_bits(v[i] * pv));
-        if constexpr (PD == AAMD_F32) prod = v[i] * pv;
-        acc[i] += prod;
+        // separate multiply and add (no FMA contraction): the reference multiplies, rounds, then sums
+        if constexpr (PD == AAMD_BF16) prod = bf16_bits_to_f32(f32_to_bf16_bits((v[i] * pv)));
+        if constexpr (PD == AAMD_F32) prod = (v[i] * pv);
+        acc[i] = acc[i] + prod;
       }
     }
     if constexpr (PD == AAMD_F32) {

@@ -46,8 +46,8 @@ template <typename IN, bool SCATTER, int U>
 __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::elem* __restrict__ x, int64_t ldx,
                                                           int nt, int64_t total_tiles,
                                                           const int32_t* __restrict__ row_map, int topk,
-                                                          uint8_t* __restrict__ q, float* __restrict__ s,
-                                                          float eps) {
+                                                          int64_t M_out, uint8_t* __restrict__ q,
+                                                          float* __restrict__ s, float eps) {
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
   const int64_t base = (int64_t)blockIdx.x * (16 * U);
   const int64_t cols = (int64_t)nt * kTile;
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     } else {
       for (int j = 0; j < topk; j++) {
         const int64_t dst = row_map[row[u] * topk + j];
-        if (dst < 0) continue;
+        if (dst < 0 || dst >= M_out) continue;
         *reinterpret_cast<v2i*>(q + dst * cols + (int64_t)tc[u] * kTile + l * 8) = codes;
         if (l == 0) s[dst * nt + tc[u]] = sc;
       }
@@ -336,14 +336,14 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   dim3 grid((unsigned)blocks), block(256);
   if (row_map == nullptr) {
     if (x_dtype == AAMD_BF16)
-      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, q, s, eps);
+      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps);
     else
-      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, q, s, eps);
+      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps);
   } else {
     if (x_dtype == AAMD_BF16)
-      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, q, s, eps);
+      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps);
     else
-      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, q, s, eps);
+      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps);
   }
   AAMD_LAUNCH_CHECK("quant_1x128");
   return AAMD_OK;
