@@ -1,0 +1,408 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 grouped-linear MoE expert path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c1]
+
+One "step" is one pass of the hot path over one synthetic routed batch, inputs already
+resident in HBM (quantised operands for the GEMM workloads, bf16 tokens for c5):
+
+  c2 (default)  Mixtral-8x7B-like expert FFN, 8 experts, hidden 4096, gate_up 2x14336 and
+                down 14336->4096, 16384 tokens top-2: the six grouped GEMMs of forward, dgrad
+                and wgrad of both layers.  metric = fp8 grouped-GEMM TFLOP/s.
+  c3            DeepSeek-V3-like, 64 experts, Zipf(1.2) ragged routing with empty groups: forward.
+  c4            Qwen-MoE-like, 60 experts, fwd + dgrad + wgrad.
+  c5            permute + 1x128 quant and unpermute + combine of 65536 x 7168 tokens (GB/s).
+  c1            the small CPU-runnable case.
+
+Prints one JSON line.  ``roofline`` prices the dominant kernel against the published MI355X
+peaks (dense fp8 MFMA 5.0 PFLOP/s, HBM 8 TB/s) from HIP-event timings taken on the launch
+stream; ``cpu_baseline`` is the reference's PyTorch CPU path (dequantise + per-expert matmul,
+or the torch quantise / permute restatement) timed on this host on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
+TILE = 128
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+# ------------------------------------------------------------------------------------------
+# synthetic routed batches (seeds fixed; generated on the device, nothing is read from disk)
+# ------------------------------------------------------------------------------------------
+def routing(T, E, k, dev, zipf_s=None, seed=2):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    if zipf_s is None:
+        logits = torch.randn(T, E, generator=g, device=dev)
+    else:
+        p = torch.arange(1, E + 1, dtype=torch.float32, device=dev).pow(-zipf_s)
+        u = torch.rand(T, E, generator=g, device=dev).clamp_min(1e-30)
+        logits = p.log() - torch.log(-torch.log(u))  # Gumbel top-k = sampling without replacement
+    vals, idx = torch.topk(logits, k, dim=1)
+    return idx, torch.softmax(vals, dim=1).to(torch.bfloat16)
+
+
+def randn(shape, dev, std, seed, dtype=torch.bfloat16):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    out = torch.empty(shape, dtype=dtype, device=dev)
+    # fill in row chunks to bound the fp32 temporary
+    rows = shape[0]
+    step = max(1, (1 << 28) // max(1, out[0].numel()))
+    for r in range(0, rows, step):
+        n = min(step, rows - r)
+        out[r : r + n] = (torch.randn((n, *shape[1:]), generator=g, device=dev) * std).to(dtype)
+    return out
+
+
+def student_t(shape, dev, seed):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    out = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+    step = max(1, (1 << 26) // shape[1])
+    for r in range(0, shape[0], step):
+        n = min(step, shape[0] - r)
+        z = torch.randn((n, shape[1]), generator=g, device=dev)
+        chi = torch.randn((n, shape[1], 3), generator=g, device=dev).pow(2).sum(-1)
+        out[r : r + n] = (z / torch.sqrt(chi / 3)).to(torch.bfloat16)
+    return out
+
+
+class Timer:
+    """HIP events on torch's current stream, which is the stream every kernel here is launched on."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def region(self):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        self.pairs.append((a, b))
+        return a, b
+
+    def ms(self):
+        return [a.elapsed_time(b) for a, b in self.pairs]
+
+
+# ------------------------------------------------------------------------------------------
+# GEMM workloads
+# ------------------------------------------------------------------------------------------
+class Layer:
+    """One grouped linear's resident operands: fp8 codes and scales of x, w, dy (+ transposes)."""
+
+    def __init__(self, kernels, M, K, N, E, goff, dev, seed, backward):
+        x = randn((M, K), dev, 1.0, seed)
+        w = randn((E, N, K), dev, 0.02, seed + 1)
+        self.M, self.K, self.N, self.E = M, K, N, E
+        self.goff = goff
+        if backward:
+            self.qx, self.sx, self.qx_t, self.sx_t = kernels.tile_quant_dual_grouped(x, goff, E)
+            dy = randn((M, N), dev, 1e-2, seed + 2)
+            self.qdy, self.sdy, self.qdy_t, self.sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E)
+            del dy
+            self.qw, self.sw, self.qw_t, self.sw_t = kernels.block_quant_batched(w, return_transpose=True)
+            self.dx = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+            self.dw = torch.empty((E, N, K), dtype=torch.float32, device=dev)
+        else:
+            self.qx, self.sx = kernels.tile_quant(x)
+            self.qw, self.sw, _, _ = kernels.block_quant_batched(w)
+        del x, w
+        self.y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        self.flops = 2.0 * M * N * K
+
+    def fwd(self, kernels):
+        kernels.grouped_gemm_nt(self.qx, self.sx, self.qw, self.sw, self.goff, out=self.y)
+
+    def dgrad(self, kernels):
+        kernels.grouped_gemm_nt(self.qdy, self.sdy, self.qw_t, self.sw_t, self.goff, out=self.dx)
+
+    def wgrad(self, kernels):
+        kernels.grouped_gemm_wgrad(self.qdy_t, self.sdy_t, self.qx_t, self.sx_t, self.goff, out=self.dw)
+
+
+GEMM_WORKLOADS = {
+    # name: (E, T, topk, zipf, [(K, N), ...], backward, description)
+    "c1": (4, 2048, 1, None, [(512, 1024)], False, "4 experts, 512->1024, 2048 tokens top-1, forward"),
+    "c2": (8, 16384, 2, None, [(4096, 28672), (14336, 4096)], True,
+           "Mixtral-8x7B-like expert FFN: 8 experts, 4096->2x14336 and 14336->4096, 16384 tokens top-2, "
+           "fwd+dgrad+wgrad"),
+    "c3": (64, 8192, 8, 1.2, [(7168, 4096), (2048, 7168)], False,
+           "DeepSeek-V3-like: 64 experts, 7168->4096 and 2048->7168, 8192 tokens top-8 Zipf(1.2), forward"),
+    "c4": (60, 32768, 4, None, [(2048, 2816), (1408, 2048)], True,
+           "Qwen-MoE-like: 60 experts, 2048->2816 and 1408->2048, 32768 tokens top-4, fwd+dgrad+wgrad"),
+}  # fmt: skip
+
+
+def run_gemm(args, kernels, dev):
+    E, T, k, zipf, shapes, backward, desc = GEMM_WORKLOADS[args.workload]
+    idx, _ = routing(T, E, k, dev, zipf_s=zipf)
+    _, _, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
+    M = T * k
+    layers = [Layer(kernels, M, K, N, E, goff, dev, 10 * i, backward) for i, (K, N) in enumerate(shapes)]
+    counts = (goff[1:] - goff[:-1]).cpu()
+    torch.cuda.synchronize()
+
+    nt_timer, wg_timer = Timer(), Timer()
+
+    def step(timed):
+        for L in layers:
+            if timed:
+                a, b = nt_timer.region()
+                a.record()
+            L.fwd(kernels)
+            if timed:
+                b.record()
+        if backward:
+            for L in layers:
+                if timed:
+                    a, b = nt_timer.region()
+                    a.record()
+                L.dgrad(kernels)
+                if timed:
+                    b.record()
+                    a, b = wg_timer.region()
+                    a.record()
+                L.wgrad(kernels)
+                if timed:
+                    b.record()
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+
+    passes = 3 if backward else 1
+    flops_step = passes * sum(L.flops for L in layers)
+    ms_step = dt * 1e3 / args.steps
+    tflops = flops_step / (ms_step * 1e-3) / 1e12
+
+    # dominant kernel: the forward / dgrad grouped GEMM (4 of the 6 launches of a step)
+    nt_ms = nt_timer.ms()
+    n_nt = len(layers) * (2 if backward else 1)
+    nt_flops = sum(L.flops for L in layers) * (2 if backward else 1) / n_nt  # per launch, averaged
+    nt_avg_ms = sum(nt_ms) / len(nt_ms)
+    nt_tflops = nt_flops / (nt_avg_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": "grouped_gemm_kernel<kRaggedRows> (forward and dgrad)",
+        "bound": "mfma",
+        "achieved": round(nt_tflops, 2),
+        "peak": PEAK_FP8_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(nt_tflops / PEAK_FP8_TFLOPS, 4),
+        "traffic": None,
+        "avg_launch_ms": round(nt_avg_ms, 4),
+        "flop_per_launch": nt_flops,
+    }
+    extras = {"tokens_per_expert_min_max": [int(counts.min()), int(counts.max())],
+              "empty_groups": int((counts == 0).sum())}
+    if backward:
+        wg_ms = wg_timer.ms()
+        wg_avg = sum(wg_ms) / len(wg_ms)
+        wg_flops = sum(L.flops for L in layers) / len(layers)
+        extras["wgrad_kernel"] = {"avg_launch_ms": round(wg_avg, 4),
+                                  "achieved_tflops": round(wg_flops / (wg_avg * 1e-3) / 1e12, 2),
+                                  "frac": round(wg_flops / (wg_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_gemm_baseline(layers[0], counts)
+    return {
+        "metric": "fp8 grouped-GEMM TFLOPS (fwd+bwd)" if backward else "fp8 grouped-GEMM TFLOPS (fwd)",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "ms_per_step": round(ms_step, 4),
+        "dtype": "fp8",
+        "config": {"workload": f"{args.workload}: {desc}", "rows": M, "experts": E,
+                   "flop_per_step": flops_step, "frac_of_fp8_peak": round(tflops / PEAK_FP8_TFLOPS, 4)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extras": extras,
+    }  # fmt: skip
+
+
+def cpu_gemm_baseline(layer, counts):
+    """The reference's PyTorch CPU path (dequantise + per-expert matmul) on a bounded sample of
+    the first layer's forward: as many leading experts as about 2e12 FLOP cover."""
+    from oracle import oracle as O
+
+    K, N = layer.K, layer.N
+    budget, rows, ne = 2.0e12, 0, 0
+    for c in counts.tolist():
+        if ne > 0 and 2.0 * (rows + c) * N * K > budget:
+            break
+        rows += c
+        ne += 1
+    if rows == 0:
+        return None
+    qx = layer.qx[:rows].view(torch.uint8).cpu()
+    sx = layer.sx[:rows].cpu()
+    qw = layer.qw[:ne].view(torch.uint8).cpu()
+    sw = layer.sw[:ne].cpu()
+    splits = counts[:ne].tolist()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    t0 = time.perf_counter()
+    ref = O.torch_grouped_gemm_dequant(qx, sx, qw, sw, splits)
+    dt = time.perf_counter() - t0
+    # the sample doubles as an end-to-end check of the GPU result
+    got = layer.y[:rows].float().cpu()
+    err = float(((got - ref.float()).abs().max()) / ref.float().abs().max().clamp_min(1e-30))
+    fl = 2.0 * rows * N * K
+    return {"value": round(fl / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"forward of layer 0, first {ne} experts ({rows} rows, {fl:.3e} FLOP, {dt:.1f} s): "
+                      "torch CPU dequantise + per-expert fp32 matmul",
+            "max_err_vs_gpu_over_max": round(err, 5)}  # fmt: skip
+
+
+# ------------------------------------------------------------------------------------------
+# c5: quant / permute kernels
+# ------------------------------------------------------------------------------------------
+def run_c5(args, kernels, dev):
+    T, H, E, k = 65536, 7168, 64, 8
+    x = student_t((T, H), dev, seed=0)
+    idx, probs = routing(T, E, k, dev)
+    _, row_map, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
+    M = T * k
+    y = randn((M, H), dev, 1.0, seed=5)
+    torch.cuda.synchronize()
+    pq_bytes = T * H * 2 + M * H + M * (H // TILE) * 4 + M * 4
+    uc_bytes = M * H * 2 + T * k * 2 + M * 4 + T * H * 2
+    tq_bytes = M * H * 2 + M * H + M * (H // TILE) * 4
+    t_pq, t_uc, t_tq, t_pre = Timer(), Timer(), Timer(), Timer()
+
+    def step(timed):
+        for timer, fn in (
+            (t_pre, lambda: kernels.moe_preprocess(idx, E, want_sorted=False)),
+            (t_pq, lambda: kernels.permute_tile_quant(x, row_map, k, M)),
+            (t_uc, lambda: kernels.unpermute_combine(y, row_map, probs, T, k)),
+            (t_tq, lambda: kernels.tile_quant(y)),
+        ):
+            if timed:
+                a, b = timer.region()
+                a.record()
+            fn()
+            if timed:
+                b.record()
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt * 1e3 / args.steps
+
+    def gbs(nbytes, timer):
+        ms = timer.ms()
+        return nbytes / (sum(ms) / len(ms) * 1e-3) / 1e9, sum(ms) / len(ms)
+
+    pq, pq_ms = gbs(pq_bytes, t_pq)
+    uc, uc_ms = gbs(uc_bytes, t_uc)
+    tq, tq_ms = gbs(tq_bytes, t_tq)
+    pre_ms = sum(t_pre.ms()) / len(t_pre.ms())
+    total_gbs = (pq_bytes + uc_bytes) / ((pq_ms + uc_ms) * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_quant_baseline(x, idx)
+    return {
+        "metric": "quant/permute HBM GB/s (permute+1x128 quant and unpermute+combine)",
+        "value": round(total_gbs, 1),
+        "unit": "GB/s",
+        "ms_per_step": round(ms_step, 4),
+        "dtype": "fp8",
+        "config": {"workload": "c5: 65536 tokens x 7168 bf16 Student-t(3), top-8 into 64 experts; "
+                               "fused permute + 1x128 quant, and unpermute + weighted combine",
+                   "rows": M, "experts": E},
+        "roofline": {"kernel": "quant_1x128_kernel<bf16, scatter> (permute + quant)", "bound": "hbm",
+                     "achieved": round(pq, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(pq / PEAK_HBM_GBS, 4), "traffic": None,
+                     "avg_launch_ms": round(pq_ms, 4), "bytes_per_launch": pq_bytes},
+        "cpu_baseline": cpu,
+        "extras": {
+            "unpermute_combine": {"GB/s": round(uc, 1), "frac": round(uc / PEAK_HBM_GBS, 4),
+                                  "avg_launch_ms": round(uc_ms, 4), "bytes_per_launch": uc_bytes},
+            "tile_quant_plain": {"GB/s": round(tq, 1), "frac": round(tq / PEAK_HBM_GBS, 4),
+                                 "avg_launch_ms": round(tq_ms, 4), "bytes_per_launch": tq_bytes},
+            "moe_preprocess_ms": round(pre_ms, 4),
+        },
+    }  # fmt: skip
+
+
+def cpu_quant_baseline(x, idx):
+    """torch CPU restatement of permute + per-row quantise on the first 2048 tokens."""
+    from oracle import oracle as O
+
+    n = 2048
+    xs = x[:n].cpu()
+    ids = idx[:n].cpu()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    t0 = time.perf_counter()
+    p, _ = O.torch_permute(xs, ids)
+    q, s = O.torch_tile_quant(p)
+    dt = time.perf_counter() - t0
+    k = ids.shape[1]
+    H = xs.shape[1]
+    nbytes = n * H * 2 + n * k * H + n * k * (H // TILE) * 4 + n * k * 4
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"first {n} tokens: torch CPU permute (argsort + index_select) then amax/448, divide, "
+                      f"cast ({dt:.2f} s)"}  # fmt: skip
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(3)
+    from atorch_amd import kernels
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
+    out = {
+        "metric": res["metric"],
+        "value": res["value"],
+        "unit": res["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": res["dtype"],
+        "data": "synthetic",
+        "config": res["config"],
+        "roofline": res["roofline"],
+        "cpu_baseline": res["cpu_baseline"],
+        "extras": res["extras"],
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -55,3 +55,65 @@ def rel_err(c: torch.Tensor, ref: torch.Tensor) -> float:
     c, ref = c.double(), ref.double()
     floor = ref.pow(2).mean().sqrt().clamp_min(1e-30)
     return float(((c - ref).abs() / torch.maximum(ref.abs(), floor)).max()) if ref.numel() else 0.0
+
+
+class OracleQuantizeOp:
+    """A ``quantize_op`` (the plugin interface of the grouped linear) that runs the CPU oracle.
+    Test infrastructure: it lets the host logic of the autograd function be checked without a
+    GPU and serves as the module-level reference on the GPU box.  Per-expert API only."""
+
+    supports_fused_grouped = False
+
+    def __init__(self):
+        from oracle import oracle as O
+
+        self.O = O
+        self.calls = {"quantize": 0, "grouped_qgemm": 0}
+
+    def quantize(self, t, qparams, return_transpose=False):
+        from atorch_amd.quantization import QuantizeResult
+
+        O = self.O
+        self.calls["quantize"] += 1
+        t = t.detach().cpu()
+        if tuple(qparams.quant_tile_shape) == (1, TILE):
+            q, s = O.tile_quant(t, qparams.eps)
+            if not return_transpose:
+                return QuantizeResult(q, s)
+            m = t.shape[0]
+            q_t, s_t = O.tile_quant_t_grouped(t, [m], qparams.eps)
+            nb = (m + TILE - 1) // TILE
+            return QuantizeResult(q, s, q_t[:, :m].contiguous(), s_t[:nb].t().contiguous())
+        q, s = O.block_quant(t, qparams.eps)
+        if not return_transpose:
+            return QuantizeResult(q, s)
+        return QuantizeResult(q, s, q.t().contiguous(), s.t().contiguous())
+
+    def grouped_qgemm(self, qa_list, qb_list, mm_params, sa_list, sb_list, out_list, bias=None, accumulate=False,
+                      qparams_x=None, qparams_w=None):
+        O = self.O
+        self.calls["grouped_qgemm"] += 1
+        wgrad = tuple(qparams_w.quant_tile_shape) == (1, TILE)
+        for e, (qa, qb, sa, sb, out) in enumerate(zip(qa_list, qb_list, sa_list, sb_list, out_list)):
+            if not wgrad:
+                if qa.shape[0] == 0:
+                    continue
+                c = O.fp8_gemm(qa.contiguous(), sa.contiguous(), qb.contiguous(), sb.contiguous())
+                if bias is not None:
+                    c = c + bias[e].float()
+                out.copy_(c.to(out.dtype))
+            else:
+                m = qa.shape[1]
+                if m == 0:
+                    if not accumulate:
+                        out.zero_()
+                    continue
+                ld = (m + TILE - 1) // TILE * TILE
+                a = torch.zeros((qa.shape[0], ld), dtype=torch.uint8)
+                b = torch.zeros((qb.shape[0], ld), dtype=torch.uint8)
+                a[:, :m], b[:, :m] = qa, qb
+                c = O.fp8_gemm(a, sa.contiguous(), b, sb.contiguous())  # b tile-scaled: sb [K, nb]
+                if accumulate:
+                    out.add_(c.to(out.dtype))
+                else:
+                    out.copy_(c.to(out.dtype))

@@ -1,0 +1,218 @@
+"""Module-level parity on the GPU, in the shape of the reference's own test
+(atorch/tests/common_tests/fp8/test_quantized_grouped_linear.py:607-737): the grouped module
+against a sequential loop of single-group modules sharing its weights (bit-wise), and against
+the CPU oracle (GEMM tolerance 1e-2); plus the gmm adapter and the dispatcher round trip."""
+import pytest
+import torch
+
+from helpers import OracleQuantizeOp, heavy_tailed, ragged_splits, randn_bf16, rel_err, topk_routing
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _run(module, x, m_splits, fuse):
+    out = module(x, m_splits)
+    out.sum().backward()
+    res = [out.detach(), x.grad.detach()]
+    for p in module.parameters():
+        if getattr(p, "main_grad", None) is not None and fuse:
+            assert p.grad is None
+            res.append(p.main_grad)
+        else:
+            res.append(p.grad)
+    return res
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("batch_size", [1, 2])
+@pytest.mark.parametrize("num_gemms", [3, 6])
+@pytest.mark.parametrize("fuse_wgrad_accumulation", [True, False])
+def test_grouped_linear_recipes(dev, dtype, batch_size, num_gemms, fuse_wgrad_accumulation, oracle):
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+
+    hidden, out_size, seq = 256, 128, 2048
+    torch.manual_seed(0)
+    grouped = ATorchGroupedLinear(num_gemms, hidden, out_size, bias=False, params_dtype=dtype, device=dev,
+                                  fuse_wgrad_accumulation=fuse_wgrad_accumulation)
+    singles = [ATorchGroupedLinear(1, hidden, out_size, bias=False, params_dtype=dtype, device=dev,
+                                   fuse_wgrad_accumulation=fuse_wgrad_accumulation) for _ in range(num_gemms)]
+    with torch.no_grad():
+        for i in range(num_gemms):
+            w = getattr(grouped, f"weight{i}")
+            singles[i].weight0.copy_(w)
+            if fuse_wgrad_accumulation:
+                w.main_grad = torch.rand_like(w, dtype=torch.float32)
+                singles[i].weight0.main_grad = w.main_grad.clone()
+    splits = ragged_splits(seq, num_gemms, seed=0, multiple=16)
+    assert 0 in splits
+    m_splits = [m * batch_size for m in splits]
+    x0 = randn_bf16((seq, batch_size, hidden), 0, dtype=dtype).to(dev)
+
+    xg = x0.clone().requires_grad_(True)
+    res = _run(grouped, xg, m_splits, fuse_wgrad_accumulation)
+
+    xs = x0.clone().requires_grad_(True)
+    outs = [singles[i](inp, [inp.shape[0] * batch_size]) for i, inp in enumerate(torch.split(xs, splits))]
+    out_seq = torch.cat(outs)
+    out_seq.sum().backward()
+    ref = [out_seq.detach(), xs.grad.detach()]
+    for s in singles:
+        p = s.weight0
+        ref.append(p.main_grad if fuse_wgrad_accumulation else p.grad)
+    # should be a bit-wise match
+    for o, r in zip(res, ref):
+        torch.testing.assert_close(o, r, rtol=0, atol=0)
+
+    # and against the CPU oracle
+    ws = [getattr(grouped, f"weight{i}").detach().cpu() for i in range(num_gemms)]
+    orc = oracle.grouped_linear_fwd_bwd(x0.cpu(), ws, m_splits, torch.ones(seq * batch_size, out_size, dtype=dtype))
+    assert rel_err(res[0].cpu().view(-1, out_size), orc["out"]) <= TOL
+    assert rel_err(res[1].cpu().view(-1, hidden), orc["dgrad"]) <= TOL
+    if not fuse_wgrad_accumulation:
+        for i in range(num_gemms):
+            assert rel_err(res[2 + i].cpu(), orc["wgrad"][i]) <= TOL
+
+
+def test_grouped_linear_bias_cache_and_nograd(dev, oracle):
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+
+    E, K, N = 4, 256, 384
+    torch.manual_seed(1)
+    mod = ATorchGroupedLinear(E, K, N, bias=True, params_dtype=torch.bfloat16, device=dev)
+    with torch.no_grad():
+        for i in range(E):
+            getattr(mod, f"bias{i}").copy_(randn_bf16((N,), 40 + i).to(dev))
+    splits = [100, 0, 313, 99]
+    x = heavy_tailed((sum(splits), K), 6).to(dev)
+    ws = [getattr(mod, f"weight{i}").detach().cpu() for i in range(E)]
+    bs = [getattr(mod, f"bias{i}").detach().cpu() for i in range(E)]
+    dy = randn_bf16((sum(splits), N), 7, std=1e-2)
+    orc = oracle.grouped_linear_fwd_bwd(x.cpu(), ws, splits, dy, biases=bs)
+    xg = x.clone().requires_grad_(True)
+    o1 = mod(xg, splits, is_first_microbatch=True)
+    o1.backward(dy.to(dev))
+    assert rel_err(o1.detach().cpu(), orc["out"]) <= TOL
+    assert rel_err(xg.grad.cpu(), orc["dgrad"]) <= TOL
+    for i in range(E):
+        assert rel_err(getattr(mod, f"weight{i}").grad.cpu(), orc["wgrad"][i]) <= TOL
+        torch.testing.assert_close(getattr(mod, f"bias{i}").grad.cpu().float(), orc["bgrad"][i], rtol=2e-2, atol=1e-3)
+    assert torch.all(mod.weight1.grad == 0)
+    # cached weights give identical results (test_quantized_grouped_linear.py:515-557)
+    o2 = mod(x, splits, is_first_microbatch=False)
+    assert torch.equal(o1.detach(), o2.detach())
+    with torch.no_grad():
+        o3 = mod(x, splits)
+    assert torch.equal(o1.detach(), o3)
+
+
+def test_plugin_list_interface_unfused_operands(dev, oracle):
+    """quantize_op.quantize per expert + grouped_qgemm on lists that do NOT tile one buffer:
+    the operator falls back to one HIP launch per group and gives the same results."""
+    from atorch_amd.quantization import HipQuantizeOp, MMParams, QParams
+
+    op = HipQuantizeOp()
+    xp, wp = QParams(quant_tile_shape=(1, 128)), QParams(quant_tile_shape=(128, 128))
+    E, K, N = 3, 256, 128
+    splits = [70, 0, 200]
+    xs = [randn_bf16((m, K), 50 + i).to(dev) for i, m in enumerate(splits)]
+    ws = [randn_bf16((N, K), 60 + i, std=0.02).to(dev) for i in range(E)]
+    dys = [randn_bf16((m, N), 70 + i, std=1e-2).to(dev) for i, m in enumerate(splits)]
+    qx = [op.quantize(x, xp, return_transpose=True) for x in xs]
+    qw = [op.quantize(w, wp, return_transpose=True) for w in ws]
+    qd = [op.quantize(d, xp, return_transpose=True) for d in dys]
+    outs = [torch.empty((m, N), dtype=torch.bfloat16, device=dev) for m in splits]
+    op.grouped_qgemm([r.data for r in qx], [r.data for r in qw], MMParams(), [r.scale for r in qx],
+                     [r.scale for r in qw], outs, qparams_x=xp, qparams_w=wp)
+    dgr = [torch.empty((m, K), dtype=torch.bfloat16, device=dev) for m in splits]
+    op.grouped_qgemm([r.data for r in qd], [r.data_t for r in qw], MMParams(), [r.scale for r in qd],
+                     [r.scale_t for r in qw], dgr, qparams_x=xp, qparams_w=wp)
+    wgr = [torch.full((N, K), 7.0, dtype=torch.float32, device=dev) for _ in range(E)]
+    op.grouped_qgemm([r.data_t for r in qd], [r.data_t for r in qx], MMParams(), [r.scale_t for r in qd],
+                     [r.scale_t for r in qx], wgr, accumulate=False, qparams_x=xp, qparams_w=xp)
+    x_all, dy_all = torch.cat(xs).cpu(), torch.cat(dys).cpu()
+    orc = oracle.grouped_linear_fwd_bwd(x_all, [w.cpu() for w in ws], splits, dy_all)
+    assert rel_err(torch.cat(outs).cpu(), orc["out"]) <= TOL
+    assert rel_err(torch.cat(dgr).cpu(), orc["dgrad"]) <= TOL
+    for e in range(E):
+        assert rel_err(wgr[e].cpu(), orc["wgrad"][e]) <= TOL
+    assert torch.all(wgr[1] == 0)
+    # the transposed results have the reference's shapes
+    assert qx[2].data_t.shape == (K, 200) and qx[2].scale_t.shape == (K, 2)
+    assert qw[0].data_t.shape == (K, N) and qw[0].scale_t.shape == (K // 128, N // 128)
+
+
+def test_module_with_oracle_operator_matches_hip_operator(dev):
+    """Same module code, two operator plugins: the HIP one on the GPU and the oracle one on the
+    CPU agree within the GEMM tolerance."""
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+    from atorch_amd.quantization import QLinearParams
+
+    E, K, N = 3, 128, 256
+    torch.manual_seed(3)
+    hip = ATorchGroupedLinear(E, K, N, bias=False, params_dtype=torch.bfloat16, device=dev)
+    cpu = ATorchGroupedLinear(E, K, N, bias=False, params_dtype=torch.bfloat16, device="cpu",
+                              qlinear_params=QLinearParams(quantize_op=OracleQuantizeOp()))
+    with torch.no_grad():
+        for i in range(E):
+            getattr(cpu, f"weight{i}").copy_(getattr(hip, f"weight{i}").cpu())
+    splits = [33, 150, 73]
+    x = randn_bf16((256, K), 9)
+    a = x.clone().to(dev).requires_grad_(True)
+    b = x.clone().requires_grad_(True)
+    oa, ob = hip(a, splits), cpu(b, splits)
+    oa.sum().backward()
+    ob.sum().backward()
+    assert rel_err(oa.detach().cpu(), ob.detach().float()) <= TOL
+    assert rel_err(a.grad.cpu(), b.grad.float()) <= TOL
+    for i in range(E):
+        assert rel_err(getattr(hip, f"weight{i}").grad.cpu(), getattr(cpu, f"weight{i}").grad.float()) <= TOL
+
+
+@pytest.mark.parametrize("trans_b", [True, False])
+def test_gmm_adapter(dev, trans_b):
+    from atorch_amd.gmm import gmm
+
+    E, K, N = 4, 256, 384
+    splits = [120, 0, 300, 92]
+    M = sum(splits)
+    a = randn_bf16((M, K), 1).to(dev).requires_grad_(True)
+    w = randn_bf16((E, N, K) if trans_b else (E, K, N), 2, std=0.02).to(dev).requires_grad_(True)
+    bs = torch.tensor(splits, dtype=torch.int64)
+    out = gmm(a, w, bs, trans_b=trans_b)
+    dy = randn_bf16((M, N), 3, std=1e-2).to(dev)
+    out.backward(dy)
+    a64 = a.detach().double().requires_grad_(True)
+    w64 = w.detach().double().requires_grad_(True)
+    outs, off = [], 0
+    for e, m in enumerate(splits):
+        we = w64[e].t() if trans_b else w64[e]
+        outs.append(a64[off : off + m] @ we)
+        off += m
+    ref = torch.cat(outs)
+    ref.backward(dy.double())
+    # against the unquantised product only quantisation noise is left (a few percent of rms)
+    def close(x, y):
+        return ((x.double() - y) ** 2).mean() <= 2e-3 * (y**2).mean() + 1e-30
+    assert out.shape == (M, N) and close(out.detach(), ref.detach())
+    assert close(a.grad, a64.grad) and close(w.grad, w64.grad)
+    assert torch.all(w.grad[1] == 0)
+
+
+def test_dispatcher_round_trip(dev, oracle):
+    from atorch_amd.token_dispatcher import MoETokenDispatcher
+
+    T, H, E, k = 500, 512, 16, 4
+    x = heavy_tailed((T, H), 12)
+    idx, probs = topk_routing(T, E, k, seed=13)
+    probs = probs.bfloat16()
+    d = MoETokenDispatcher(E, k)
+    permuted, goff = d.token_permutation(x.to(dev), probs.to(dev), idx.to(dev))
+    xp, so, counts = oracle.permute(x, idx, E)
+    assert torch.equal(permuted.cpu(), xp)
+    assert torch.equal((goff[1:] - goff[:-1]).cpu(), counts)
+    out, _ = d.token_unpermutation(permuted)
+    assert torch.equal(out.cpu(), oracle.unpermute(xp, so, probs))
+    q, s, goff2 = d.token_permutation_fp8(x.to(dev), probs.to(dev), idx.to(dev))
+    qo, sco = oracle.tile_quant(xp)
+    assert torch.equal(q.view(torch.uint8).cpu(), qo) and torch.equal(s.cpu(), sco)
