@@ -62,6 +62,13 @@ def tile_quant(
     rows = x.numel() // cols if cols else 0
     if return_transpose:
         assert x.dim() == 2, "return_transpose needs a 2-D input"
+        if rows == 0:  # an empty group: nothing to launch
+            return (
+                torch.empty((0, cols), dtype=FP8, device=x.device),
+                torch.empty((0, cols // TILE), dtype=torch.float32, device=x.device),
+                torch.empty((cols, 0), dtype=FP8, device=x.device),
+                torch.empty((cols, 0), dtype=torch.float32, device=x.device),
+            )
         goff = torch.tensor([0, rows], dtype=torch.int64, device=x.device)
         y, s, y_t, s_t = tile_quant_dual_grouped(x, goff, 1, eps=eps, ld_t=padded_total([rows]))
         return y, s, y_t[:, :rows], s_t.t()
