@@ -8,17 +8,22 @@
 //   R = the operand whose row index ends up on the MFMA row / register axis
 //       (forward+dgrad: the weight rows of the group's expert; wgrad: the rows of X^T).
 //
-// Output is C[l, r] with r contiguous, so the four consecutive MFMA rows a lane owns are
-// four consecutive output elements.  A workgroup of 256 threads (4 waves, 2x2) computes a
-// 128 x 128 tile; each wave a 64 x 64 sub-tile as 4 x 4 v_mfma_f32_16x16x128_f8f6f4 (one MFMA
-// = one full 128-deep scale block, so the raw dot product never needs a second instruction).
-// The raw product is folded into the fp32 accumulator with the scales of that block:
+// Output is C[l, r] with r contiguous, so the four consecutive MFMA rows a lane owns are four
+// consecutive output elements.  The contraction advances in steps of 128 bytes = one scale
+// block.  Per step and 32x32 sub-tile two chained v_mfma_f32_32x32x64_f8f6f4 give the raw
+// 128-deep dot products, which are folded into the fp32 accumulator with the step's scales:
 //   acc += p * (l_scale[l, kb] * r_scale)      r_scale per 128x128 block (one scalar) or per row.
-// The per-lane l_scale sits in a VGPR because the L row is the lane axis.
+// The per-lane l_scale sits in one VGPR because the L row is the lane axis.
 //
-// Tiles of 128 contraction bytes are staged global -> VGPR -> LDS (double buffered, one
-// barrier per step) with an XOR swizzle of the 16-byte chunks so that both the 16-byte
-// stores and the MFMA operand reads are bank-conflict free.
+// Why this shape of MFMA: measured on MI355X, VALU instructions co-execute with the 16-pass
+// 32x32x64 MFMA (8 FMAs per MFMA cost ~4 %), but not with the 8-pass 16x16x128 one (there every
+// FMA adds its full 4 cycles).  The fold needs 8 FMAs per MFMA, so only the former keeps the
+// matrix pipe busy.
+//
+// Data path: global -> LDS directly (global_load_lds, 16 bytes per lane, no register stop),
+// two stages, one workgroup barrier per step.  Rows are 128 bytes; the 16-byte chunks of a row
+// are XOR-swizzled so that the linear 1 KB writes of the direct loads and the 32-row MFMA
+// operand reads are both bank-conflict free on the 64-bank LDS (measured: ~235 of 256 B/clk).
 #include <stdlib.h>
 
 #include "common.hpp"
@@ -29,11 +34,12 @@ constexpr int kBK = 128;  // contraction bytes per step == scale block
 
 enum GemmMode { kRaggedRows = 0, kRaggedK = 1 };
 
-// XOR swizzle of the 16-byte chunk index inside a 128-byte LDS row.
-#ifndef AAMD_SWZ_SHIFT
-#define AAMD_SWZ_SHIFT 1
-#endif
-__device__ __forceinline__ int swz(int row) { return (row >> AAMD_SWZ_SHIFT) & 7; }
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// XOR swizzle of the 16-byte chunk index inside a 128-byte LDS row (depends on row % 16 only).
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 struct GemmParams {
   const uint8_t* L;
@@ -43,7 +49,7 @@ struct GemmParams {
   void* C;
   const void* bias;
   const int64_t* goff;      // [E+1] rows per group prefix (device); nullptr: one group [0, Lrows)
-  const int32_t* tile_off;  // [E+1] 128-row tile prefix (device)
+  const int32_t* tile_off;  // [E+1] tile prefix (device)
   int64_t ldl, ldr;                          // row strides of L and R (bytes)
   int64_t r_group_stride;                    // bytes between the R matrices of consecutive groups
   int64_t ls_row_stride, ls_blk_stride;      // L scale (row, block) strides, floats
@@ -54,29 +60,23 @@ struct GemmParams {
   int64_t Rrows;   // rows of R per group
   int nkb;         // kRaggedRows: K / 128
   int E;
-  int nRt;         // Rrows / 128
-  int nLt;         // kRaggedK: Lrows / 128
+  int nRt;         // R tiles
+  int nLt;         // kRaggedK: L tiles
   int max_kb;      // kRaggedK: contraction blocks the operand buffers hold (ld_t / 128)
   int accumulate;
   int bias_dtype;
 };
 
-__device__ __forceinline__ v4f mfma_fp8_16x16x128(const v8i& a, const v8i& b) {
-  const v4f z = {0.f, 0.f, 0.f, 0.f};
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, z, 0, 0, 0, 0, 0, 0);
+__device__ __forceinline__ v16f mfma_fp8_32x32x64(const v8i& a, const v8i& b, const v16f& c) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
 template <typename OUT>
-__device__ __forceinline__ void store4(OUT* dst, const v4f& v, bool accumulate) {
+__device__ __forceinline__ void store4(OUT* dst, v4f o, bool accumulate) {
   if constexpr (sizeof(OUT) == 4) {
-    v4f o = v;
-    if (accumulate) {
-      const v4f old = *reinterpret_cast<const v4f*>(dst);
-      o += old;
-    }
+    if (accumulate) o += *reinterpret_cast<const v4f*>(dst);
     *reinterpret_cast<v4f*>(dst) = o;
   } else {
-    v4f o = v;
     if (accumulate) {
       const v2i old = *reinterpret_cast<const v2i*>(dst);
       o[0] += bf16_bits_to_f32((uint32_t)old[0] & 0xffffu);
@@ -91,20 +91,23 @@ __device__ __forceinline__ void store4(OUT* dst, const v4f& v, bool accumulate) 
   }
 }
 
-// Tile configuration: WR x WL waves, each computing (WTR*16) R rows x (WTL*16) L rows.
+// Tile configuration: WR x WL waves, each computing (WTR*32) R rows x (WTL*32) L rows.
 template <int WR_, int WL_, int WTR_, int WTL_>
 struct Cfg {
   static constexpr int WR = WR_, WL = WL_, WTR = WTR_, WTL = WTL_;
   static constexpr int NT = 64 * WR * WL;   // threads
-  static constexpr int BM = WL * WTL * 16;  // L rows per workgroup tile
-  static constexpr int BN = WR * WTR * 16;  // R rows per workgroup tile
+  static constexpr int BM = WL * WTL * 32;  // L rows per workgroup tile
+  static constexpr int BN = WR * WTR * 32;  // R rows per workgroup tile
   static constexpr int LCH = BM * 8 / NT;   // 16-byte chunks per thread and step (L)
   static constexpr int RCH = BN * 8 / NT;
   static_assert(NT >= BM + BN, "one thread per scale value");
-  static_assert((WTR * 16) % 128 == 0 || BN == 128, "a wave's R rows stay inside one 128-row scale block");
+  static_assert(BM % 64 == 0 && BN % 128 == 0, "whole waves per scale side; R tiles cover whole scale blocks");
+  static_assert((WTR * 32) % 128 == 0 || BN == 128, "a wave's R rows stay inside one 128-row scale block");
+  static_assert(LCH * NT == BM * 8 && RCH * NT == BN * 8, "tile rows divide evenly over the threads");
 };
-typedef Cfg<2, 2, 4, 4> CfgSmall;  // 256 threads, 128 x 128
-typedef Cfg<2, 4, 8, 4> CfgLarge;  // 512 threads, 256 x 256
+typedef Cfg<2, 2, 2, 2> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two workgroups per CU
+typedef Cfg<2, 4, 4, 2> CfgLarge;  // 512 threads, 256 (L) x 256 (R)
+typedef Cfg<2, 4, 2, 2> CfgWgrad;  // 512 threads, 256 (L) x 128 (R): room for the per-row R scales
 
 // A 64-bit offset the compiler can keep in scalar registers (it is the same in every lane).
 __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
@@ -116,9 +119,10 @@ __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
 template <int MODE, bool R_PER_ROW, typename OUT, typename C>
 __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kernel(const GemmParams p) {
   constexpr int BM = C::BM, BN = C::BN, NT = C::NT;
-  __shared__ __attribute__((aligned(16))) uint8_t Lbuf[2][BM * kBK];
-  __shared__ __attribute__((aligned(16))) uint8_t Rbuf[2][BN * kBK];
-  __shared__ __attribute__((aligned(16))) float Sc[2][BM + BN];  // [buf][L rows | R rows or R blocks]
+  // two stages as separate arrays: loads into one are known not to alias reads of the other
+  __shared__ __attribute__((aligned(16))) uint8_t Lbuf0[BM * kBK], Lbuf1[BM * kBK];
+  __shared__ __attribute__((aligned(16))) uint8_t Rbuf0[BN * kBK], Rbuf1[BN * kBK];
+  __shared__ __attribute__((aligned(16))) float Sc0[NT], Sc1[NT];  // [L rows | R rows or R blocks | unused]
   __shared__ int slot;
 
   const int tid = threadIdx.x;
@@ -185,160 +189,217 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   const float* Lsg = p.Ls + (int64_t)kb0 * p.ls_blk_stride;
   const float* Rsg = p.Rs + (int64_t)g * p.rs_group_stride + (int64_t)kb0 * p.rs_blk_stride;
 
-  // ---- global -> register staging: LCH + RCH chunks of 16 bytes per thread -----------------
-  const int ld_row = tid >> 3, ld_ch = tid & 7;
-  int loff[C::LCH], roff[C::RCH], lds_loff[C::LCH], lds_roff[C::RCH];
+  // ---- global -> LDS without a register stop ---------------------------------------------------
+  // One wave instruction of the direct load writes 1 KB of LDS, lane l at base + 16 l: eight
+  // tile rows of 128 bytes.  Lane l owns LDS position (row l/8, chunk l%8) and fetches the
+  // global chunk the swizzle assigns to that position.
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+  const int lane = tid & 63;
+  const int ld_row = tid >> 3, ld_pch = tid & 7;
+  uint32_t loff[C::LCH], roff[C::RCH];  // unsigned 32-bit offsets from the uniform tile bases
 #pragma unroll
   for (int n = 0; n < C::LCH; n++) {
     const int row = ld_row + (NT / 8) * n;
     const int lrow = row < lvalid ? row : lvalid - 1;
-    loff[n] = lrow * (int)p.ldl + ld_ch * 16;
-    lds_loff[n] = row * kBK + ((ld_ch ^ swz(row)) << 4);
+    loff[n] = (uint32_t)lrow * (uint32_t)p.ldl + (uint32_t)((ld_pch ^ swz(row)) << 4);
   }
 #pragma unroll
   for (int n = 0; n < C::RCH; n++) {
     const int row = ld_row + (NT / 8) * n;
     const int rrow = row < rvalid ? row : rvalid - 1;
-    roff[n] = rrow * (int)p.ldr + ld_ch * 16;
-    lds_roff[n] = row * kBK + ((ld_ch ^ swz(row)) << 4);
+    roff[n] = (uint32_t)rrow * (uint32_t)p.ldr + (uint32_t)((ld_pch ^ swz(row)) << 4);
   }
   // scales: thread t < BM fetches the L scale of row t; thread BM + t the R scale of row t
-  // (per-row scales) or of 128-row block t (block scales)
-  const float* sptr = Lsg + l0 * p.ls_row_stride;  // threads without a scale re-read a valid one
-  int64_t s_step = 0;
-  if (tid < BM) {
+  // (per-row scales) or of 128-row block t (block scales); the rest re-read a valid value.
+  // Whole waves are on one side (BM is a multiple of 64), so base and step are wave-uniform.
+  const bool l_side = wave < BM / 64;
+  const float* sbase = l_side ? Lsg + l0 * p.ls_row_stride : Rsg + (R_PER_ROW ? r0 : r0 / kTile) * p.rs_row_stride;
+  const int64_t s_step = l_side ? p.ls_blk_stride : p.rs_blk_stride;
+  uint32_t soff;  // element offset of this thread's scale from sbase
+  if (l_side) {
     const int lrow = tid < lvalid ? tid : lvalid - 1;
-    sptr = Lsg + (l0 + lrow) * p.ls_row_stride;
-    s_step = p.ls_blk_stride;
-  } else if (tid < BM + BN) {
+    soff = (uint32_t)lrow * (uint32_t)p.ls_row_stride;
+  } else {
     const int t = tid - BM;
-    if (R_PER_ROW) {
-      const int rrow = t < rvalid ? t : rvalid - 1;
-      sptr = Rsg + (r0 + rrow) * p.rs_row_stride;
-      s_step = p.rs_blk_stride;
-    } else if (t < BN / kTile) {
-      const int blk = t * kTile < rvalid ? t : rvalid / kTile - 1;
-      sptr = Rsg + (r0 / kTile + blk) * p.rs_row_stride;
-      s_step = p.rs_blk_stride;
-    }
+    const int nvalid = R_PER_ROW ? rvalid : rvalid / kTile;
+    const int rr = t < nvalid ? t : nvalid - 1;
+    soff = (uint32_t)rr * (uint32_t)p.rs_row_stride;
   }
-  const int s_slot = tid < BM + BN ? tid : 0;  // NT == BM + BN for the shipped configurations
 
-  v4i lreg[C::LCH], rreg[C::RCH];
-  float sreg = 0.f;
-  auto g_load = [&](int kb) {
+  // touch-ahead: thread t < BM owns L row t, thread BM + t owns R row t (clamped like the loads)
+#ifndef AAMD_TOUCH_AHEAD
+#define AAMD_TOUCH_AHEAD 0
+#endif
+  constexpr int kTouchAhead = AAMD_TOUCH_AHEAD;
+  const uint8_t* tbase = l_side ? Lbase : Rbase;
+  uint32_t toff;
+  if (l_side) {
+    const int lrow = tid < lvalid ? tid : lvalid - 1;
+    toff = (uint32_t)lrow * (uint32_t)p.ldl;
+  } else {
+    const int t = tid - BM;
+    const int rrow = t < rvalid ? t : rvalid - 1;
+    toff = (uint32_t)rrow * (uint32_t)p.ldr;
+  }
+
+  // All loads of the contraction loop are issued from inline assembly, with the wait counts kept
+  // by hand: the compiler's own bookkeeping of direct-to-LDS loads is conservative (it tracks
+  // eight of them individually and otherwise waits for every outstanding load, including the
+  // touch loads that are meant to stay in flight).  Per step and thread: LCH + RCH 16-byte tile
+  // loads, one 4-byte scale load, one 4-byte touch load; all of them write LDS only, so no VGPR
+  // is ever written behind the compiler's back.
+  auto lds_addr = [](const void* q) { return (uint32_t)(uintptr_t)(lds_ptr_t)q; };
+  __shared__ uint32_t trash[64];  // landing zone of the touch loads, never read
+  const uint32_t trash_lds = lds_addr(trash);
+  const uint32_t soff_b = soff * 4u;
+  auto dma = [&](int kb, uint8_t* Ld, uint8_t* Rd, float* Sd) {
     const uint8_t* lb = Lbase + (int64_t)kb * kBK;
     const uint8_t* rb = Rbase + (int64_t)kb * kBK;
+    const uint8_t* sb = reinterpret_cast<const uint8_t*>(sbase + (int64_t)kb * s_step);
 #pragma unroll
-    for (int n = 0; n < C::LCH; n++) lreg[n] = *reinterpret_cast<const v4i*>(lb + loff[n]);
+    for (int n = 0; n < C::LCH; n++)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   ::"v"(loff[n]), "s"(lb), "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
+                   : "memory");
 #pragma unroll
-    for (int n = 0; n < C::RCH; n++) rreg[n] = *reinterpret_cast<const v4i*>(rb + roff[n]);
-    sreg = sptr[(int64_t)kb * s_step];
+    for (int n = 0; n < C::RCH; n++)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   ::"v"(roff[n]), "s"(rb), "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
+                   : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 ::"v"(soff_b), "s"(sb), "s"(lds_addr(Sd) + (uint32_t)(wave * 256))
+                 : "memory");
+    // Touch the cache lines of a later step (one 128-byte line per tile row and thread) so that
+    // the L2 misses of that step are already in flight: a step cannot start before its slowest
+    // line has arrived, and two LDS stages alone do not cover an HBM round trip.
+    const int kp = kb + kTouchAhead < nkb ? kb + kTouchAhead : nkb - 1;
+    const uint8_t* tb = tbase + (int64_t)kp * kBK;
+    if constexpr (kTouchAhead > 0)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(toff), "s"(tb), "s"(trash_lds)
+                   : "memory");
   };
-  auto s_store = [&](int buf) {
-#pragma unroll
-    for (int n = 0; n < C::LCH; n++) *reinterpret_cast<v4i*>(&Lbuf[buf][lds_loff[n]]) = lreg[n];
-#pragma unroll
-    for (int n = 0; n < C::RCH; n++) *reinterpret_cast<v4i*>(&Rbuf[buf][lds_roff[n]]) = rreg[n];
-    Sc[buf][s_slot] = sreg;
+  // End of a step: everything but the newest touch load has landed, then the workgroup barrier.
+  auto dma_wait_and_sync = [&]() {
+    if constexpr (kTouchAhead > 0)
+      asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
 
   // ---- MFMA tiling ------------------------------------------------------------------------
-  const int wave = tid >> 6, lane = tid & 63;
+  // v_mfma_f32_32x32x64_f8f6f4: lane l supplies operand row l%32 and 32 contraction bytes chosen
+  // by l/32; with two MFMAs per 128-byte step a lane reads, per row and K half h, the logical
+  // chunks 4h + 2(l/32) and 4h + 2(l/32) + 1.  Any assignment works as long as L and R use the
+  // same one.  D: lane l holds column l%32, rows 8(r/4) + 4(l/32) + r%4 for r = 0..15.
   const int wr = wave / C::WL, wl = wave % C::WL;
-  const int l16 = lane & 15, lg = lane >> 4;
-  const int sw = swz(l16);
-  const int ch0 = ((2 * lg) ^ sw) << 4, ch1 = ((2 * lg + 1) ^ sw) << 4;
-  const int wrow0 = wr * C::WTR * 16;            // first R row of this wave inside the tile
-  const int wlrow0 = wl * C::WTL * 16;           // first L row of this wave inside the tile
+  const int l32 = lane & 31, hg = lane >> 5;
+  const int sw = swz(l32);
+  int chk[2][2];  // byte offset of the two chunks of K half h inside this lane's row
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) chk[h][c] = ((4 * h + 2 * hg + c) ^ sw) << 4;
+  const int wrow0 = wr * C::WTR * 32;            // first R row of this wave inside the tile
+  const int wlrow0 = wl * C::WTL * 32;           // first L row of this wave inside the tile
   const bool wave_active = wrow0 < rvalid;        // whole wave in or out: rvalid % 128 == 0
 
-  v4f acc[C::WTR][C::WTL];
+  v16f acc[C::WTR][C::WTL];
 #pragma unroll
   for (int i = 0; i < C::WTR; i++)
 #pragma unroll
-    for (int j = 0; j < C::WTL; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < C::WTL; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  if (nkb > 0) {
-    g_load(0);
-    s_store(0);
-  }
-  __syncthreads();
-
-  // Software pipeline inside the wave, pinned with scheduling barriers: the MFMA of sub-tile t
-  // is issued, then the four scale-and-accumulate FMAs of sub-tile t-1 run in its shadow (the
-  // waves of a workgroup move in lock step between barriers, so MFMA and VALU work must
-  // overlap inside one wave, not across waves).  The loop body is branch free: the prefetch of
-  // the last step re-reads the last block, and waves outside a partial R tile compute on
-  // clamped rows and skip only the final store.
-  for (int kb = 0; kb < nkb; kb++) {
-    const int cur = kb & 1;
-    g_load(kb + 1 < nkb ? kb + 1 : kb);
-
-    const uint8_t* Lt = Lbuf[cur];
-    const uint8_t* Rt = Rbuf[cur];
-    const float* Lsc = &Sc[cur][0];
-    const float* Rsc = &Sc[cur][BM];
-    v8i lf[C::WTL];
+  // One 128-deep step on the stage (Lt, Rt, Sct).  Per 32x32 sub-tile t: two chained MFMAs, then
+  // the 16 scale-and-accumulate FMAs of sub-tile t-1 run in their shadow.  The wanted issue
+  // order is described to the scheduler with group barriers and fenced with scheduling
+  // barriers; the accumulators are tied to the end of the step so the FMAs cannot drift past
+  // the workgroup barrier.  Branch free: waves outside a partial R tile compute on clamped
+  // rows and skip only the final store.
+  constexpr int NTILES = C::WTR * C::WTL;
+  auto compute = [&](const uint8_t* Lt, const uint8_t* Rt, const float* Sct) {
+    __builtin_amdgcn_sched_barrier(0);
+    const float* Lsc = Sct;
+    const float* Rsc = Sct + BM;
+    auto load_frag = [&](const uint8_t* T, int row, int h) {
+      const v4i lo = *reinterpret_cast<const v4i*>(T + row * kBK + chk[h][0]);
+      const v4i hi = *reinterpret_cast<const v4i*>(T + row * kBK + chk[h][1]);
+      return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    v8i lf[C::WTL][2];
     float cs[C::WTL];
     const float rblk = R_PER_ROW ? 1.f : Rsc[wrow0 / kTile];
 #pragma unroll
     for (int j = 0; j < C::WTL; j++) {
-      const int row = wlrow0 + j * 16 + l16;
-      const v4i lo = *reinterpret_cast<const v4i*>(Lt + row * kBK + ch0);
-      const v4i hi = *reinterpret_cast<const v4i*>(Lt + row * kBK + ch1);
-      lf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      const int row = wlrow0 + j * 32 + l32;
+      lf[j][0] = load_frag(Lt, row, 0);
+      lf[j][1] = load_frag(Lt, row, 1);
       cs[j] = Lsc[row] * rblk;
     }
-    auto load_rf = [&](int i) {
-      const int row = wrow0 + i * 16 + l16;
-      const v4i lo = *reinterpret_cast<const v4i*>(Rt + row * kBK + ch0);
-      const v4i hi = *reinterpret_cast<const v4i*>(Rt + row * kBK + ch1);
-      return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    };
-    auto load_rs = [&](int i) {
-      v4f r = {1.f, 1.f, 1.f, 1.f};
-      if constexpr (R_PER_ROW) r = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 16 + 4 * lg]);
-      return r;
-    };
-    v8i rf[2];
-    v4f rs4[2];
-    rf[0] = load_rf(0);
-    rs4[0] = load_rs(0);
-    v4f pprev = {0.f, 0.f, 0.f, 0.f};
-    __builtin_amdgcn_sched_barrier(0);
+    v8i rf[2][2];
+    v4f rs[2][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
+    auto load_r = [&](int i) {
+      const int row = wrow0 + i * 32 + l32;
+      rf[i & 1][0] = load_frag(Rt, row, 0);
+      rf[i & 1][1] = load_frag(Rt, row, 1);
+      if constexpr (R_PER_ROW) {
 #pragma unroll
-    for (int i = 0; i < C::WTR; i++) {
-#pragma unroll
-      for (int j = 0; j < C::WTL; j++) {
-        const v4f pcur = mfma_fp8_16x16x128(rf[i & 1], lf[j]);
-        if (i > 0 || j > 0) {
-          const int pi = j > 0 ? i : i - 1, pj = j > 0 ? j - 1 : C::WTL - 1;
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const float sc = R_PER_ROW ? cs[pj] * rs4[pi & 1][r] : cs[pj];
-            acc[pi][pj][r] = __builtin_fmaf(pprev[r], sc, acc[pi][pj][r]);
-          }
-        }
-        pprev = pcur;
-        // the fragments of the next R row tile are fetched once the last FMA that needed the
-        // previous row tile's scales has been placed
-        if (j == 0 && i + 1 < C::WTR) {
-          rf[(i + 1) & 1] = load_rf(i + 1);
-          rs4[(i + 1) & 1] = load_rs(i + 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        for (int q = 0; q < 4; q++)
+          rs[i & 1][q] = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 32 + 8 * q + 4 * hg]);
       }
-    }
+    };
+    v16f pr[2];
+    load_r(0);
+    auto fold = [&](int t) {  // acc of sub-tile t += raw product * scales
+      const int i = t / C::WTL, j = t % C::WTL;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const float sc = R_PER_ROW ? cs[C::WTL - 1] * rs4[(C::WTR - 1) & 1][r] : cs[C::WTL - 1];
-      acc[C::WTR - 1][C::WTL - 1][r] = __builtin_fmaf(pprev[r], sc, acc[C::WTR - 1][C::WTL - 1][r]);
+      for (int r = 0; r < 16; r++) {
+        const float sc = R_PER_ROW ? cs[j] * rs[i & 1][r / 4][r % 4] : cs[j];
+        acc[i][j][r] = __builtin_fmaf(pr[t & 1][r], sc, acc[i][j][r]);
+      }
+    };
+    v16f zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NTILES; t++) {
+      const int i = t / C::WTL, j = t % C::WTL;
+      pr[t & 1] = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
+      pr[t & 1] = mfma_fp8_32x32x64(rf[i & 1][1], lf[j][1], pr[t & 1]);
+      if (t >= 1) fold(t - 1);
+      // the next row of R sub-tiles is fetched once the fold that still needed the scales in
+      // the slot it overwrites (the last sub-tile of the previous row) has been placed
+      if (j == 0 && i + 1 < C::WTR) load_r(i + 1);
     }
+    fold(NTILES - 1);
+#pragma unroll
+    for (int t = 0; t < NTILES; t++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
+      if (t % C::WTL == 0) __builtin_amdgcn_sched_group_barrier(0x100, R_PER_ROW ? 8 : 4, 0);  // LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x002, R_PER_ROW ? 32 : 16, 0);  // VALU of the previous sub-tile
+    }
+    // tie the accumulators to this point: the FMAs above may not drift past the barrier below
+#pragma unroll
+    for (int i = 0; i < C::WTR; i++)
+#pragma unroll
+      for (int j = 0; j < C::WTL; j++) asm volatile("" : "+v"(acc[i][j]));
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-    s_store(cur ^ 1);
-    __syncthreads();
+  if (nkb > 0) dma(0, Lbuf0, Rbuf0, Sc0);
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  int kb = 0;
+  for (; kb + 1 < nkb; kb += 2) {  // two steps per trip, the stages swap roles
+    dma(kb + 1, Lbuf1, Rbuf1, Sc1);
+    compute(Lbuf0, Rbuf0, Sc0);
+    dma_wait_and_sync();
+    dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
+    compute(Lbuf1, Rbuf1, Sc1);
+    dma_wait_and_sync();
   }
+  if (kb < nkb) compute(Lbuf0, Rbuf0, Sc0);  // odd number of steps
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the touch loads
 
   // ---- epilogue ------------------------------------------------------------------------------
   if (MODE == kRaggedK && nkb == 0 && p.accumulate) return;  // empty group: leave dW untouched
@@ -346,23 +407,27 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   OUT* Cg = reinterpret_cast<OUT*>(p.C) + (int64_t)g * p.c_group_stride;
 #pragma unroll
   for (int i = 0; i < C::WTR; i++) {
-    const int64_t rcol = r0 + wrow0 + i * 16 + 4 * lg;
-    v4f b4 = {0.f, 0.f, 0.f, 0.f};
-    if (MODE == kRaggedRows && p.bias != nullptr) {
-      if (p.bias_dtype == AAMD_F32) {
-        b4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(p.bias) + g * p.bias_group_stride + rcol);
-      } else {
-        const v2i raw = *reinterpret_cast<const v2i*>(reinterpret_cast<const u16*>(p.bias) + g * p.bias_group_stride + rcol);
-        b4[0] = bf16_bits_to_f32((uint32_t)raw[0] & 0xffffu);
-        b4[1] = bf16_bits_to_f32((uint32_t)raw[0] >> 16);
-        b4[2] = bf16_bits_to_f32((uint32_t)raw[1] & 0xffffu);
-        b4[3] = bf16_bits_to_f32((uint32_t)raw[1] >> 16);
-      }
-    }
 #pragma unroll
-    for (int j = 0; j < C::WTL; j++) {
-      const int lrow = wlrow0 + j * 16 + l16;
-      if (lrow < lvalid) store4<OUT>(Cg + (l0 + lrow) * p.ldc + rcol, acc[i][j] + b4, p.accumulate != 0);
+    for (int q = 0; q < 4; q++) {
+      const int64_t rcol = r0 + wrow0 + i * 32 + 8 * q + 4 * hg;
+      v4f b4 = {0.f, 0.f, 0.f, 0.f};
+      if (MODE == kRaggedRows && p.bias != nullptr) {
+        if (p.bias_dtype == AAMD_F32) {
+          b4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(p.bias) + g * p.bias_group_stride + rcol);
+        } else {
+          const v2i raw = *reinterpret_cast<const v2i*>(reinterpret_cast<const u16*>(p.bias) + g * p.bias_group_stride + rcol);
+          b4[0] = bf16_bits_to_f32((uint32_t)raw[0] & 0xffffu);
+          b4[1] = bf16_bits_to_f32((uint32_t)raw[0] >> 16);
+          b4[2] = bf16_bits_to_f32((uint32_t)raw[1] & 0xffffu);
+          b4[3] = bf16_bits_to_f32((uint32_t)raw[1] >> 16);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < C::WTL; j++) {
+        const int lrow = wlrow0 + j * 32 + l32;
+        const v4f o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        if (lrow < lvalid) store4<OUT>(Cg + (l0 + lrow) * p.ldc + rcol, o + b4, p.accumulate != 0);
+      }
     }
   }
 }
@@ -387,8 +452,10 @@ static bool use_large_tiles(int64_t l_rows, int64_t r_rows, int64_t groups) {
   const char* env = getenv("AAMD_GEMM_TILE");
   if (env && env[0] == 's') return false;
   if (env && env[0] == 'l') return true;
-  const int64_t tiles = ((l_rows + 255) / 256) * ((r_rows + 255) / 256) * groups;
-  return tiles >= 512;
+  // Measured on MI355X at the Mixtral expert shapes the 128x128 configuration (two workgroups per
+  // CU) is the faster one; the 256-wide configurations stay selectable for experiments.
+  (void)l_rows; (void)r_rows; (void)groups;
+  return false;
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -414,9 +481,12 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
   AAMD_REQUIRE(lda >= K && lda % 16 == 0 && aligned16(a) && aligned16(b), "grouped_gemm_nt: operands must be 16-byte aligned");
   AAMD_REQUIRE(ldc >= N && ldc % 4 == 0 && aligned16(c), "grouped_gemm_nt: output must be 16-byte aligned");
   AAMD_REQUIRE(K > 0, "grouped_gemm_nt: K must be positive");
+  AAMD_REQUIRE(lda < (1LL << 23) && K < (1LL << 23), "grouped_gemm_nt: row stride too large");
   hipStream_t st = (hipStream_t)stream;
+  // tile-scaled B carries per-row R scales: use the configuration that has room for them
   const bool large = use_large_tiles(M, N, 1);
-  const int BM = large ? CfgLarge::BM : CfgSmall::BM, BN = large ? CfgLarge::BN : CfgSmall::BN;
+  const int BM = large ? CfgLarge::BM : CfgSmall::BM;
+  const int BN = large ? (b_tile_scaled ? CfgWgrad::BN : CfgLarge::BN) : CfgSmall::BN;
   if (group_offsets) {
     int rc = launch_group_tile_offsets(group_offsets, E, BM, tile_ws, st);
     if (rc) return rc;
@@ -435,7 +505,7 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
   const int64_t max_lt = group_offsets ? M / BM + E : (M + BM - 1) / BM;
   const int64_t blocks = max_lt * p.nRt;
   if (large)
-    return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgLarge>(p, c_dtype, blocks, st)
+    return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgWgrad>(p, c_dtype, blocks, st)
                          : launch_gemm<kRaggedRows, false, CfgLarge>(p, c_dtype, blocks, st);
   return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgSmall>(p, c_dtype, blocks, st)
                        : launch_gemm<kRaggedRows, false, CfgSmall>(p, c_dtype, blocks, st);
@@ -450,6 +520,7 @@ extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt
                "grouped_gemm_wgrad: N=%lld and K=%lld must be multiples of 128", (long long)N, (long long)K);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "grouped_gemm_wgrad: group_offsets / tile_ws required");
   AAMD_REQUIRE(ld_t >= 0 && ld_t % kBK == 0, "grouped_gemm_wgrad: ld_t=%lld must be a multiple of 128", (long long)ld_t);
+  AAMD_REQUIRE(ld_t < (1LL << 23), "grouped_gemm_wgrad: ld_t too large");
   if (N == 0 || K == 0) return AAMD_OK;
   AAMD_REQUIRE(dw && (ld_t == 0 || (dyt && sdyt && xt && sxt)), "grouped_gemm_wgrad: null pointer");
   AAMD_REQUIRE(aligned16(dyt) && aligned16(xt) && aligned16(dw), "grouped_gemm_wgrad: pointers must be 16-byte aligned");
@@ -465,11 +536,11 @@ extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt
   p.bias = nullptr; p.bias_dtype = AAMD_NONE; p.bias_group_stride = 0;
   p.goff = group_offsets; p.tile_off = tile_ws;
   const bool large = use_large_tiles(N, K, E);
-  const int BM = large ? CfgLarge::BM : CfgSmall::BM, BN = large ? CfgLarge::BN : CfgSmall::BN;
+  const int BM = large ? CfgWgrad::BM : CfgSmall::BM, BN = large ? CfgWgrad::BN : CfgSmall::BN;
   p.Lrows = N; p.Rrows = K; p.nkb = 0; p.E = E; p.nRt = (int)((K + BN - 1) / BN); p.nLt = (int)((N + BM - 1) / BM);
   p.max_kb = (int)(ld_t / kBK);
   p.accumulate = accumulate;
   const int64_t blocks = (int64_t)E * p.nLt * p.nRt;
-  return large ? launch_gemm<kRaggedK, true, CfgLarge>(p, dw_dtype, blocks, st)
+  return large ? launch_gemm<kRaggedK, true, CfgWgrad>(p, dw_dtype, blocks, st)
                : launch_gemm<kRaggedK, true, CfgSmall>(p, dw_dtype, blocks, st);
 }
