@@ -33,6 +33,11 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
 TILE = 128
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# this file (with --copy-probe: a plain 1 GiB copy reads FETCH_SIZE*2.0 KiB, WRITE_SIZE*1.0 KiB), averaged
+# over that kernel's launches of one step.  Counters cannot be read from inside the process, so the
+# figures are recorded here beside the profile summaries they come from (profiles/*.txt).
+MEASURED_TRAFFIC_BYTES = {"c2": 17.8e9, "c5": 4.857e9}
 
 
 def parse():
@@ -42,7 +47,19 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one plain 1 GiB device-to-device copy before the timed region: under "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its known size calibrates the counters")
     return ap.parse_args()
+
+
+def copy_probe(dev):
+    """A plain copy of known size (1 GiB read + 1 GiB written) for counter calibration."""
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
 
 
 # ------------------------------------------------------------------------------------------
@@ -208,7 +225,7 @@ def run_gemm(args, kernels, dev):
         "peak": PEAK_FP8_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(nt_tflops / PEAK_FP8_TFLOPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
         "avg_launch_ms": round(nt_avg_ms, 4),
         "flop_per_launch": nt_flops,
     }
@@ -336,7 +353,7 @@ def run_c5(args, kernels, dev):
                    "rows": M, "experts": E},
         "roofline": {"kernel": "quant_1x128_kernel<bf16, scatter> (permute + quant)", "bound": "hbm",
                      "achieved": round(pq, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(pq / PEAK_HBM_GBS, 4), "traffic": None,
+                     "frac": round(pq / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c5"),
                      "avg_launch_ms": round(pq_ms, 4), "bytes_per_launch": pq_bytes},
         "cpu_baseline": cpu,
         "extras": {
@@ -382,6 +399,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.copy_probe:
+        copy_probe(dev)
     res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
     out = {
         "metric": res["metric"],
