@@ -362,10 +362,9 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
   AAMD_REQUIRE((q == nullptr) == (s == nullptr), "quant_dual: q and s go together");
   AAMD_REQUIRE(q_t && s_t, "quant_dual: q_t / s_t required");
   if (cols == 0) return AAMD_OK;
-  // sum_g ceil(M_g/128) <= floor(M/128) + E; the caller's ld_t must hold the real total,
-  // which only the device knows: every tile beyond ld_t/128 would be out of bounds, so the
-  // grid is clamped to ld_t/128 padded tiles and ld_t is required to cover the upper bound
-  // whenever the bound is what the caller used.
+  // The padded tile count sum_g ceil(M_g/128) is known only on the device; floor(M/128) + E bounds
+  // it.  The grid covers min(bound, ld_t/128) tiles, so no tile can land beyond column ld_t of the
+  // transposed outputs; tiles past the real total find no group and exit.
   const int64_t max_tiles = M / kTile + E;
   const int64_t grid_tiles = ld_t / kTile < max_tiles ? ld_t / kTile : max_tiles;
   if (grid_tiles == 0) return AAMD_OK;

@@ -12,7 +12,29 @@
  * pin it against torch's CPU cast over all 2^16 bf16 patterns and against an
  * exact rational-arithmetic rounder.
  *
- * Parity status per function (what pins it) is listed in oracle/README.md.
+ * Parity status: what pins each function (tests/test_oracle.py, tests/test_golden.py)
+ *   oracle_f32_to_e4m3fn / oracle_e4m3fn_to_f32   pinned: torch's CPU cast on all 2^16 bf16 patterns and
+ *       10^6 random fp32 values, an exact rational rounder on ties / subnormals / the 448-464-465 edge,
+ *       round trip over all 256 codes
+ *   f32_to_bf16                                   pinned: torch's cast on 2*10^5 random values
+ *   oracle_tile_quant / oracle_block_quant        pinned: closed form s = fl(max(amax,eps)/448) and exact
+ *       rational rounding of fl(x/s); the reference tests' known answers (zeros, ones, 1000, -512, the 1e4
+ *       outlier); independent torch restatement; error bound; transpose and row-permutation invariants
+ *   oracle_tile_quant_t_grouped                   pinned: equals tile quant of the zero padded transpose of
+ *       each group (torch restatement), partial tiles and empty groups included
+ *   oracle_fp8_gemm                               pinned: float64 dequantise-and-matmul (library routine),
+ *       pure-Python brute force in the reference's accumulation order, linearity / accumulate,
+ *       grouped == per-expert loop, fp64 autograd of the unquantised problem (roles and transposes)
+ *   oracle_permute_indices                        pinned: torch.argsort(stable=True), bincount
+ *   oracle_unpermute_combine                      pinned: brute force, torch restatement (index_copy_,
+ *       multiply, sum) bit-exact for bf16 weights, inverse-of-permute property
+ * Parity unpinned (nothing available here can pin it; the oracle's choice is stated instead):
+ *   - the exact fp32 rounding of the reference's compiled Triton division x / s on its GPU: the oracle
+ *     is defined as IEEE round-to-nearest division;
+ *   - the numerics and layouts of the external `kitchen` package behind quantize_op (not in the
+ *     reference tree, no version pinned): the in-tree Triton formulas are the anchor instead;
+ *   - the summation order of torch's GPU `sum(dim=1)` in unpermute for fp32 weights: the oracle sums the
+ *     top-k terms sequentially in fp32.
  *
  * Build: gcc -O2 -fno-fast-math -ffp-contract=off -shared -fPIC (see Makefile).
  */
