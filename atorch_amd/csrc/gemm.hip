@@ -65,6 +65,7 @@ struct GemmParams {
   int max_kb;      // kRaggedK: contraction blocks the operand buffers hold (ld_t / 128)
   int accumulate;
   int bias_dtype;
+  int gl;          // L tiles that share an R panel in the tile order
 };
 
 __device__ __forceinline__ v16f mfma_fp8_32x32x64(const v8i& a, const v8i& b, const v16f& c) {
@@ -92,9 +93,11 @@ __device__ __forceinline__ void store4(OUT* dst, v4f o, bool accumulate) {
 }
 
 // Tile configuration: WR x WL waves, each computing (WTR*32) R rows x (WTL*32) L rows.
-template <int WR_, int WL_, int WTR_, int WTL_>
+template <int WR_, int WL_, int WTR_, int WTL_, int PRB_ = 2, bool LAHEAD_ = false>
 struct Cfg {
+  static constexpr bool LAHEAD = LAHEAD_;  // load the L tile two steps ahead (extra barrier per step)
   static constexpr int WR = WR_, WL = WL_, WTR = WTR_, WTL = WTL_;
+  static constexpr int PRB = PRB_;  // raw-product buffers: 2 folds a sub-tile under the next one's MFMAs
   static constexpr int NT = 64 * WR * WL;   // threads
   static constexpr int BM = WL * WTL * 32;  // L rows per workgroup tile
   static constexpr int BN = WR * WTR * 32;  // R rows per workgroup tile
@@ -104,9 +107,16 @@ struct Cfg {
   static_assert(BM % 64 == 0 && BN % 128 == 0, "whole waves per scale side; R tiles cover whole scale blocks");
   static_assert((WTR * 32) % 128 == 0 || BN == 128, "a wave's R rows stay inside one 128-row scale block");
   static_assert(LCH * NT == BM * 8 && RCH * NT == BN * 8, "tile rows divide evenly over the threads");
+  static_assert((NT / 8) % 16 == 0, "the swizzle of a slab depends on the wave only");
 };
-typedef Cfg<2, 2, 2, 2> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two workgroups per CU
-typedef Cfg<2, 4, 4, 2> CfgLarge;  // 512 threads, 256 (L) x 256 (R)
+typedef Cfg<2, 2, 2, 2, 3> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two workgroups per CU
+#ifndef AAMD_LARGE_PRB
+#define AAMD_LARGE_PRB 1
+#endif
+#ifndef AAMD_LARGE_LAHEAD
+#define AAMD_LARGE_LAHEAD true
+#endif
+typedef Cfg<2, 4, 4, 2, AAMD_LARGE_PRB, AAMD_LARGE_LAHEAD> CfgLarge;  // 512 threads, 256 (L) x 256 (R); one product buffer: 256 registers per lane
 typedef Cfg<2, 4, 2, 2> CfgWgrad;  // 512 threads, 256 (L) x 128 (R): room for the per-row R scales
 
 // A 64-bit offset the compiler can keep in scalar registers (it is the same in every lane).
@@ -119,35 +129,51 @@ __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
 template <int MODE, bool R_PER_ROW, typename OUT, typename C>
 __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kernel(const GemmParams p) {
   constexpr int BM = C::BM, BN = C::BN, NT = C::NT;
-  // two stages as separate arrays: loads into one are known not to alias reads of the other
-  __shared__ __attribute__((aligned(16))) uint8_t Lbuf0[BM * kBK], Lbuf1[BM * kBK];
-  __shared__ __attribute__((aligned(16))) uint8_t Rbuf0[BN * kBK], Rbuf1[BN * kBK];
-  __shared__ __attribute__((aligned(16))) float Sc0[NT], Sc1[NT];  // [L rows | R rows or R blocks | unused]
+  // LDS: two stages, each [L tile | R tile] of 128-byte rows, then the two stages' scales
+  // ([L rows | R rows or R blocks | unused], NT floats each).  After the contraction loop the same
+  // memory stages the output tile for the row-contiguous stores of the epilogue.
+  constexpr int kStage = (BM + BN) * kBK;
+  constexpr int kStgBytes = 64 * 144;  // per-wave epilogue staging: 64 rows x (128 + 16) bytes
+  static_assert(2 * kStage >= (NT / 64) * kStgBytes, "the epilogue staging fits in the stage buffers");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4];
   __shared__ int slot;
+  uint8_t* const Lbuf0 = lds;
+  uint8_t* const Rbuf0 = lds + BM * kBK;
+  uint8_t* const Lbuf1 = lds + kStage;
+  uint8_t* const Rbuf1 = lds + kStage + BM * kBK;
+  float* const Sc0 = reinterpret_cast<float*>(lds + 2 * kStage);
+  float* const Sc1 = Sc0 + NT;
 
   const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+  const int lane = tid & 63;
 
-  // ---- which tile -------------------------------------------------------------------
-  // Workgroup ids go round-robin over the 8 XCDs; give every XCD one contiguous range of
-  // tile ids so that tiles sharing operand panels meet in the same L2.
+  // ---- which tile -------------------------------------------------------------------------
+  // One tile per workgroup (a loop over tiles inside the kernel costs registers and the
+  // hardware's own dispatch balances ragged tiles better).  Workgroup ids go round-robin over
+  // the 8 XCDs; every XCD gets one contiguous range of tile ids so that tiles sharing operand
+  // panels meet in the same L2.
+  const int total_lt = MODE == kRaggedRows ? (p.goff ? p.tile_off[p.E] : (int)((p.Lrows + BM - 1) / BM))
+                                           : p.nLt * p.E;
+  const int64_t ntot = (int64_t)total_lt * p.nRt;
+  const int64_t bid = blockIdx.x;
+  if (bid >= ntot) return;
   int g, lt, rt;
   {
-    const int total_lt = MODE == kRaggedRows ? (p.goff ? p.tile_off[p.E] : (int)((p.Lrows + BM - 1) / BM))
-                                             : p.nLt * p.E;
-    const int64_t ntot = (int64_t)total_lt * p.nRt;
-    const int64_t bid = blockIdx.x;
-    if (bid >= ntot) return;
     const int64_t per = ntot / 8, rem = ntot % 8;
     const int64_t xcd = bid % 8, idx = bid / 8;
     const int64_t pid = xcd < rem ? xcd * (per + 1) + idx : rem * (per + 1) + (xcd - rem) * per + idx;
     // inside the range: groups of GL L tiles, R tile index outer, L tile inner
-    constexpr int GL = 8;
+    const int GL = p.gl;
     const int64_t width = (int64_t)GL * p.nRt;
     const int first = (int)(pid / width) * GL;
     const int gsz = total_lt - first < GL ? total_lt - first : GL;
     const int in_grp = (int)(pid % width);
     lt = first + in_grp % gsz;
     rt = in_grp / gsz;
+#if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE == 3
+    lt = 0; rt = 0;  // measurement build: every workgroup streams the same tile
+#endif
   }
 
   int64_t l0;     // first L row of the tile
@@ -193,21 +219,33 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // One wave instruction of the direct load writes 1 KB of LDS, lane l at base + 16 l: eight
   // tile rows of 128 bytes.  Lane l owns LDS position (row l/8, chunk l%8) and fetches the
   // global chunk the swizzle assigns to that position.
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
-  const int lane = tid & 63;
-  const int ld_row = tid >> 3, ld_pch = tid & 7;
-  uint32_t loff[C::LCH], roff[C::RCH];  // unsigned 32-bit offsets from the uniform tile bases
+  // A wave instruction n covers the 8-row slab starting at tile row wave*8 + (NT/8)*n.  The lane
+  // part of the address (row inside the slab, swizzled chunk) is the same for every slab of a
+  // wave: (row & 7) is lane/8 and ((row >> 3) & 1) is wave & 1 because NT/8 is a multiple of 16.
+  // The slab part is wave-uniform and lives in scalar registers.  Rows past the valid part of a
+  // tile are never stored, so they may read whatever follows them in the operand; only the end
+  // of the operand itself must not be crossed: slabs beyond the last readable row are moved onto
+  // the last slab that holds one, and that slab clamps its rows per lane.
+  const int r8 = lane >> 3;
+  const uint32_t chunk = (uint32_t)(((lane & 7) ^ r8 ^ (wave & 1)) << 4);
+  const int64_t l_rows_left = p.Lrows - l0;
+  const int availL = l_rows_left < BM ? (int)l_rows_left : BM;  // >= 1
+  const int bmaxL = ((availL - 1) >> 3) << 3, tailL = availL - bmaxL;
+  const uint32_t voffL = (uint32_t)r8 * (uint32_t)p.ldl + chunk;
+  const uint32_t voffLt = (uint32_t)(r8 < tailL ? r8 : tailL - 1) * (uint32_t)p.ldl + chunk;
+  const uint32_t voffR = (uint32_t)r8 * (uint32_t)p.ldr + chunk;  // rvalid is a multiple of 128: whole slabs
+  uint32_t lslab[C::LCH], rslab[C::RCH];  // scalar byte offsets of the slabs
+  bool ltail[C::LCH];
 #pragma unroll
   for (int n = 0; n < C::LCH; n++) {
-    const int row = ld_row + (NT / 8) * n;
-    const int lrow = row < lvalid ? row : lvalid - 1;
-    loff[n] = (uint32_t)lrow * (uint32_t)p.ldl + (uint32_t)((ld_pch ^ swz(row)) << 4);
+    const int b = wave * 8 + (NT / 8) * n;
+    ltail[n] = b >= bmaxL;
+    lslab[n] = __builtin_amdgcn_readfirstlane((uint32_t)(ltail[n] ? bmaxL : b) * (uint32_t)p.ldl);
   }
 #pragma unroll
   for (int n = 0; n < C::RCH; n++) {
-    const int row = ld_row + (NT / 8) * n;
-    const int rrow = row < rvalid ? row : rvalid - 1;
-    roff[n] = (uint32_t)rrow * (uint32_t)p.ldr + (uint32_t)((ld_pch ^ swz(row)) << 4);
+    const int b = wave * 8 + (NT / 8) * n;
+    rslab[n] = __builtin_amdgcn_readfirstlane((uint32_t)(b < rvalid ? b : rvalid - 8) * (uint32_t)p.ldr);
   }
   // scales: thread t < BM fetches the L scale of row t; thread BM + t the R scale of row t
   // (per-row scales) or of 128-row block t (block scales); the rest re-read a valid value.
@@ -226,64 +264,56 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     soff = (uint32_t)rr * (uint32_t)p.rs_row_stride;
   }
 
-  // touch-ahead: thread t < BM owns L row t, thread BM + t owns R row t (clamped like the loads)
-#ifndef AAMD_TOUCH_AHEAD
-#define AAMD_TOUCH_AHEAD 0
-#endif
-  constexpr int kTouchAhead = AAMD_TOUCH_AHEAD;
-  const uint8_t* tbase = l_side ? Lbase : Rbase;
-  uint32_t toff;
-  if (l_side) {
-    const int lrow = tid < lvalid ? tid : lvalid - 1;
-    toff = (uint32_t)lrow * (uint32_t)p.ldl;
-  } else {
-    const int t = tid - BM;
-    const int rrow = t < rvalid ? t : rvalid - 1;
-    toff = (uint32_t)rrow * (uint32_t)p.ldr;
-  }
-
   // All loads of the contraction loop are issued from inline assembly, with the wait counts kept
   // by hand: the compiler's own bookkeeping of direct-to-LDS loads is conservative (it tracks
-  // eight of them individually and otherwise waits for every outstanding load, including the
-  // touch loads that are meant to stay in flight).  Per step and thread: LCH + RCH 16-byte tile
-  // loads, one 4-byte scale load, one 4-byte touch load; all of them write LDS only, so no VGPR
-  // is ever written behind the compiler's back.
+  // eight of them individually and otherwise waits for every outstanding load).  Per step and
+  // thread: LCH + RCH 16-byte tile loads and one 4-byte scale load; all of them write LDS only,
+  // so no VGPR is ever written behind the compiler's back.
   auto lds_addr = [](const void* q) { return (uint32_t)(uintptr_t)(lds_ptr_t)q; };
-  __shared__ uint32_t trash[64];  // landing zone of the touch loads, never read
-  const uint32_t trash_lds = lds_addr(trash);
   const uint32_t soff_b = soff * 4u;
-  auto dma = [&](int kb, uint8_t* Ld, uint8_t* Rd, float* Sd) {
-    const uint8_t* lb = Lbase + (int64_t)kb * kBK;
-    const uint8_t* rb = Rbase + (int64_t)kb * kBK;
+#ifdef AAMD_GEMM_NOSCALE
+  constexpr int kScaleLd = 0;  // measurement build: no scale loads
+#else
+  constexpr int kScaleLd = 1;
+#endif
+  auto dma_scale = [&](int kb, float* Sd) {
     const uint8_t* sb = reinterpret_cast<const uint8_t*>(sbase + (int64_t)kb * s_step);
+    if constexpr (kScaleLd)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                   ::"v"(soff_b), "s"(sb), "s"(lds_addr(Sd) + (uint32_t)(wave * 256))
+                   : "memory");
+  };
+  // L half of a step: the L tile and, from the waves that own them, the L scales.
+  auto dmaL = [&](int kb, uint8_t* Ld, float* Sd) {
+    const uint8_t* lb = Lbase + (int64_t)kb * kBK;
 #pragma unroll
     for (int n = 0; n < C::LCH; n++)
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   ::"v"(loff[n]), "s"(lb), "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
+                   ::"v"(ltail[n] ? voffLt : voffL), "s"(lb + lslab[n]),
+                     "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
                    : "memory");
+    if (l_side) dma_scale(kb, Sd);
+  };
+  auto dmaR = [&](int kb, uint8_t* Rd, float* Sd) {
+    const uint8_t* rb = Rbase + (int64_t)kb * kBK;
 #pragma unroll
     for (int n = 0; n < C::RCH; n++)
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   ::"v"(roff[n]), "s"(rb), "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
+                   ::"v"(voffR), "s"(rb + rslab[n]),
+                     "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
                    : "memory");
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 ::"v"(soff_b), "s"(sb), "s"(lds_addr(Sd) + (uint32_t)(wave * 256))
-                 : "memory");
-    // Touch the cache lines of a later step (one 128-byte line per tile row and thread) so that
-    // the L2 misses of that step are already in flight: a step cannot start before its slowest
-    // line has arrived, and two LDS stages alone do not cover an HBM round trip.
-    const int kp = kb + kTouchAhead < nkb ? kb + kTouchAhead : nkb - 1;
-    const uint8_t* tb = tbase + (int64_t)kp * kBK;
-    if constexpr (kTouchAhead > 0)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(toff), "s"(tb), "s"(trash_lds)
-                   : "memory");
+    if (!l_side) dma_scale(kb, Sd);
   };
-  // End of a step: everything but the newest touch load has landed, then the workgroup barrier.
+  auto dma = [&](int kb, uint8_t* Ld, uint8_t* Rd, float* Sd) {
+    dmaL(kb, Ld, Sd);
+    dmaR(kb, Rd, Sd);
+  };
+  // End of a step: this thread's loads have landed, then the workgroup barrier.
   auto dma_wait_and_sync = [&]() {
-    if constexpr (kTouchAhead > 0)
-      asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE >= 4
+    return;  // measurement build: no waits, no barriers
+#endif
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
 
   // ---- MFMA tiling ------------------------------------------------------------------------
@@ -318,11 +348,14 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // the workgroup barrier.  Branch free: waves outside a partial R tile compute on clamped
   // rows and skip only the final store.
   constexpr int NTILES = C::WTR * C::WTL;
-  auto compute = [&](const uint8_t* Lt, const uint8_t* Rt, const float* Sct) {
+  auto compute = [&](const uint8_t* Lt, const uint8_t* Rt, const float* Sct, auto&& after_l_reads) {
     __builtin_amdgcn_sched_barrier(0);
     const float* Lsc = Sct;
     const float* Rsc = Sct + BM;
     auto load_frag = [&](const uint8_t* T, int row, int h) {
+#if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE >= 5
+      { v8i f; asm volatile("" : "=v"(f)); return f; }  // measurement build: operands from nowhere
+#endif
       const v4i lo = *reinterpret_cast<const v4i*>(T + row * kBK + chk[h][0]);
       const v4i hi = *reinterpret_cast<const v4i*>(T + row * kBK + chk[h][1]);
       return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -349,35 +382,54 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
           rs[i & 1][q] = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 32 + 8 * q + 4 * hg]);
       }
     };
-    v16f pr[2];
+    // raw-product buffers: sub-tile t's fold runs D = PRB - 1 sub-tiles later (0: right after it).
+    // Per-row R scales live in a two-slot ring that allows at most D = 1.
+    constexpr int PRB = R_PER_ROW && C::PRB > 2 ? 2 : C::PRB;
+    constexpr int D = PRB - 1;
+    v16f pr[PRB];
     load_r(0);
-    auto fold = [&](int t) {  // acc of sub-tile t += raw product * scales
+    __builtin_amdgcn_sched_barrier(0);
+    after_l_reads();  // the L fragments and L scales of this step are on their way to registers
+    __builtin_amdgcn_sched_barrier(0);
+    // acc of sub-tile t += raw product * scales, registers [8*half, 8*half + 8) of the sub-tile
+    auto fold_half = [&](int t, int half) {
       const int i = t / C::WTL, j = t % C::WTL;
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
+      for (int r = 8 * half; r < 8 * half + 8; r++) {
         const float sc = R_PER_ROW ? cs[j] * rs[i & 1][r / 4][r % 4] : cs[j];
-        acc[i][j][r] = __builtin_fmaf(pr[t & 1][r], sc, acc[i][j][r]);
+        acc[i][j][r] = __builtin_fmaf(pr[t % PRB][r], sc, acc[i][j][r]);
       }
     };
     v16f zero;
 #pragma unroll
     for (int r = 0; r < 16; r++) zero[r] = 0.f;
+    // Issue order per sub-tile, kept by full scheduling barriers: first MFMA, half of the previous
+    // sub-tile's fold, second MFMA, the other half, then the LDS reads of the next R row.  Each MFMA
+    // (16 passes) covers its own issue plus eight FMAs of another sub-tile.
 #pragma unroll
     for (int t = 0; t < NTILES; t++) {
       const int i = t / C::WTL, j = t % C::WTL;
-      pr[t & 1] = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
-      pr[t & 1] = mfma_fp8_32x32x64(rf[i & 1][1], lf[j][1], pr[t & 1]);
-      if (t >= 1) fold(t - 1);
-      // the next row of R sub-tiles is fetched once the fold that still needed the scales in
-      // the slot it overwrites (the last sub-tile of the previous row) has been placed
+      __builtin_amdgcn_sched_barrier(0);
+      pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
+      __builtin_amdgcn_sched_barrier(0);
+      if (D >= 1 && t >= D) fold_half(t - D, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][1], lf[j][1], pr[t % PRB]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (D >= 1 && t >= D) fold_half(t - D, 1);
+      if (D == 0) {
+        fold_half(t, 0);
+        fold_half(t, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // the next R row overwrites the fragment and scale slot of row i - 1, whose last fold is done
       if (j == 0 && i + 1 < C::WTR) load_r(i + 1);
     }
-    fold(NTILES - 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < NTILES; t++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
-      if (t % C::WTL == 0) __builtin_amdgcn_sched_group_barrier(0x100, R_PER_ROW ? 8 : 4, 0);  // LDS reads
-      __builtin_amdgcn_sched_group_barrier(0x002, R_PER_ROW ? 32 : 16, 0);  // VALU of the previous sub-tile
+    for (int t = NTILES - D; t < NTILES; t++) {
+      fold_half(t, 0);
+      fold_half(t, 1);
     }
     // tie the accumulators to this point: the FMAs above may not drift past the barrier below
 #pragma unroll
@@ -387,56 +439,156 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  if (nkb > 0) dma(0, Lbuf0, Rbuf0, Sc0);
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  int kb = 0;
-  for (; kb + 1 < nkb; kb += 2) {  // two steps per trip, the stages swap roles
-    dma(kb + 1, Lbuf1, Rbuf1, Sc1);
-    compute(Lbuf0, Rbuf0, Sc0);
-    dma_wait_and_sync();
-    dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
-    compute(Lbuf1, Rbuf1, Sc1);
-    dma_wait_and_sync();
+  // Measurement builds only: AAMD_GEMM_ABLATE=1 issues no loads inside the loop, =2 skips the MFMA
+  // work, to time the two halves of the pipeline separately.  Results are wrong in both.
+#ifndef AAMD_GEMM_ABLATE
+#define AAMD_GEMM_ABLATE 0
+#endif
+  constexpr bool kLoads = AAMD_GEMM_ABLATE != 1 && AAMD_GEMM_ABLATE < 4, kMath = AAMD_GEMM_ABLATE < 2 || AAMD_GEMM_ABLATE >= 4;
+  auto nothing = [] {};
+  if constexpr (!C::LAHEAD) {
+    if (nkb > 0) dma(0, Lbuf0, Rbuf0, Sc0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    int kb = 0;
+    for (; kb + 1 < nkb; kb += 2) {  // two steps per trip, the stages swap roles
+      if (kLoads) dma(kb + 1, Lbuf1, Rbuf1, Sc1);
+      if (kMath) compute(Lbuf0, Rbuf0, Sc0, nothing);
+      dma_wait_and_sync();
+      if (kLoads) dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
+      if (kMath) compute(Lbuf1, Rbuf1, Sc1, nothing);
+      dma_wait_and_sync();
+    }
+    if (kb < nkb) compute(Lbuf0, Rbuf0, Sc0, nothing);  // odd number of steps
+  } else {
+    // The L fragments of a step sit in registers for the whole step, so the L half of a stage is
+    // free as soon as every wave has read it: an extra barrier after those reads lets the L tile of
+    // step k+2 start two steps ahead, and only the R tile of step k+1 has a single step to arrive.
+    // Loads complete in issue order, so "all but the newest L group" is one wait count.  Past the
+    // end the loads re-read the last block to keep the counts uniform.
+    auto kclamp = [&](int k) { return k < nkb ? k : nkb - 1; };
+    auto wait_all_but_newest_l = [&]() {
+      if (l_side) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
+      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
+    };
+    if (nkb > 0) {
+      dmaL(0, Lbuf0, Sc0);
+      dmaR(0, Rbuf0, Sc0);
+      dmaL(kclamp(1), Lbuf1, Sc1);
+      wait_all_but_newest_l();
+      for (int kb = 0; kb < nkb; kb++) {
+        uint8_t* Lc = kb & 1 ? Lbuf1 : Lbuf0;
+        uint8_t* Rc = kb & 1 ? Rbuf1 : Rbuf0;
+        uint8_t* Rn = kb & 1 ? Rbuf0 : Rbuf1;
+        float* Sc = kb & 1 ? Sc1 : Sc0;
+        float* Sn = kb & 1 ? Sc0 : Sc1;
+        if (kLoads) dmaR(kclamp(kb + 1), Rn, Sn);
+        auto mid = [&]() {
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
+          if (kLoads) dmaL(kclamp(kb + 2), Lc, Sc);
+        };
+        if (kMath) compute(Lc, Rc, Sc, mid);
+        else mid();
+        if (kLoads) wait_all_but_newest_l();
+        else asm volatile("s_barrier" ::: "memory");
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
+    }
   }
-  if (kb < nkb) compute(Lbuf0, Rbuf0, Sc0);  // odd number of steps
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the touch loads
 
   // ---- epilogue ------------------------------------------------------------------------------
+  // A lane holds, for one output row, groups of four consecutive columns; stored directly that
+  // would be 8-byte pieces in 32 different rows per instruction.  Each wave instead transposes its
+  // tile through its own LDS region and writes 128-byte row segments: 8 lanes x 16 bytes per row.
   if (MODE == kRaggedK && nkb == 0 && p.accumulate) return;  // empty group: leave dW untouched
+  __syncthreads();  // every wave is done with the stage buffers
   if (!wave_active) return;
   OUT* Cg = reinterpret_cast<OUT*>(p.C) + (int64_t)g * p.c_group_stride;
+  uint8_t* const stg = lds + wave * kStgBytes;
+  constexpr int WROWS = C::WTL * 32;
+  static_assert(WROWS == 64, "the staging region holds 64 rows");
+  auto flush = [&](auto tag) {
+    using ST = decltype(tag);  // staging type: OUT, or float when the old output is added in fp32
+    constexpr int CW = 128 / (int)sizeof(ST);  // columns per chunk
+    constexpr int SUBS = CW / 32;              // 32-column sub-tiles per chunk
+    constexpr int PITCH = 128 + (sizeof(ST) == 2 ? 8 : 16);
+    constexpr int VL = 16 / (int)sizeof(ST);   // columns per lane in the store phase
+    static_assert(C::WTR % SUBS == 0, "chunks cover whole sub-tiles");
 #pragma unroll
-  for (int i = 0; i < C::WTR; i++) {
+    for (int ci = 0; ci < C::WTR / SUBS; ci++) {
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const int64_t rcol = r0 + wrow0 + i * 32 + 8 * q + 4 * hg;
-      v4f b4 = {0.f, 0.f, 0.f, 0.f};
-      if (MODE == kRaggedRows && p.bias != nullptr) {
-        if (p.bias_dtype == AAMD_F32) {
-          b4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(p.bias) + g * p.bias_group_stride + rcol);
-        } else {
-          const v2i raw = *reinterpret_cast<const v2i*>(reinterpret_cast<const u16*>(p.bias) + g * p.bias_group_stride + rcol);
-          b4[0] = bf16_bits_to_f32((uint32_t)raw[0] & 0xffffu);
-          b4[1] = bf16_bits_to_f32((uint32_t)raw[0] >> 16);
-          b4[2] = bf16_bits_to_f32((uint32_t)raw[1] & 0xffffu);
-          b4[3] = bf16_bits_to_f32((uint32_t)raw[1] >> 16);
+      for (int si = 0; si < SUBS; si++) {
+        const int i = ci * SUBS + si;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int64_t rcol = r0 + wrow0 + i * 32 + 8 * q + 4 * hg;
+          v4f b4 = {0.f, 0.f, 0.f, 0.f};
+          if (MODE == kRaggedRows && p.bias != nullptr) {
+            if (p.bias_dtype == AAMD_F32) {
+              b4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(p.bias) + g * p.bias_group_stride + rcol);
+            } else {
+              const v2i raw = *reinterpret_cast<const v2i*>(reinterpret_cast<const u16*>(p.bias) + g * p.bias_group_stride + rcol);
+              b4[0] = bf16_bits_to_f32((uint32_t)raw[0] & 0xffffu);
+              b4[1] = bf16_bits_to_f32((uint32_t)raw[0] >> 16);
+              b4[2] = bf16_bits_to_f32((uint32_t)raw[1] & 0xffffu);
+              b4[3] = bf16_bits_to_f32((uint32_t)raw[1] >> 16);
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < C::WTL; j++) {
+            const v4f o = v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]} + b4;
+            uint8_t* dst = stg + (j * 32 + l32) * PITCH + (si * 32 + 8 * q + 4 * hg) * (int)sizeof(ST);
+            if constexpr (sizeof(ST) == 4) {
+              *reinterpret_cast<v4f*>(dst) = o;
+            } else {
+              v2i w;
+              w[0] = (int)(f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16));
+              w[1] = (int)(f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16));
+              *reinterpret_cast<v2i*>(dst) = w;
+            }
+          }
         }
       }
+      __builtin_amdgcn_wave_barrier();  // same wave, in-order LDS: the reads below see the writes above
+      const int64_t col = r0 + wrow0 + ci * CW + (lane & 7) * VL;
 #pragma unroll
-      for (int j = 0; j < C::WTL; j++) {
-        const int lrow = wlrow0 + j * 32 + l32;
-        const v4f o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-        if (lrow < lvalid) store4<OUT>(Cg + (l0 + lrow) * p.ldc + rcol, o + b4, p.accumulate != 0);
+      for (int ps = 0; ps < WROWS / 8; ps++) {
+        const int row = ps * 8 + (lane >> 3);
+        const int lrow = wlrow0 + row;
+        const v4i raw = *reinterpret_cast<const v4i*>(stg + row * PITCH + (lane & 7) * 16);
+        if (lrow < lvalid) {
+          OUT* out = Cg + (l0 + lrow) * p.ldc + col;
+          if constexpr (sizeof(ST) == sizeof(OUT)) {
+            if constexpr (sizeof(OUT) == 4) {
+              v4f o = __builtin_bit_cast(v4f, raw);
+              if (p.accumulate) o += *reinterpret_cast<const v4f*>(out);
+              *reinterpret_cast<v4f*>(out) = o;
+            } else {
+              *reinterpret_cast<v4i*>(out) = raw;
+            }
+          } else {  // fp32 staging, bf16 output with accumulation
+            store4<OUT>(out, __builtin_bit_cast(v4f, raw), true);
+          }
+        }
       }
+      __builtin_amdgcn_wave_barrier();  // the next chunk overwrites the region
     }
+  };
+  if constexpr (sizeof(OUT) == 4) {
+    flush(float{});
+  } else {
+    if (p.accumulate) flush(float{});
+    else flush(u16{});
   }
 }
 
 int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st);
 
 template <int MODE, bool R_PER_ROW, typename C>
-static int launch_gemm(const GemmParams& p, int c_dtype, int64_t blocks, hipStream_t st) {
+static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st) {
   if (blocks <= 0) return AAMD_OK;
+  p.gl = 8;
+  if (const char* env = getenv("AAMD_GEMM_GL")) p.gl = atoi(env) > 0 ? atoi(env) : 8;
+
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "grouped_gemm: grid too large");
   dim3 grid((unsigned)blocks), block(C::NT);
   if (c_dtype == AAMD_BF16)
@@ -448,14 +600,14 @@ static int launch_gemm(const GemmParams& p, int c_dtype, int64_t blocks, hipStre
 }
 
 // Large tiles whenever the problem has enough of them to fill the chip; AAMD_GEMM_TILE=small|large overrides.
-static bool use_large_tiles(int64_t l_rows, int64_t r_rows, int64_t groups) {
+// Tile choice.  AAMD_GEMM_TILE=small|large overrides it (for experiments and tests).
+static bool use_large_tiles(int64_t tiles_256, bool by_default) {
   const char* env = getenv("AAMD_GEMM_TILE");
   if (env && env[0] == 's') return false;
   if (env && env[0] == 'l') return true;
-  // Measured on MI355X at the Mixtral expert shapes the 128x128 configuration (two workgroups per
-  // CU) is the faster one; the 256-wide configurations stay selectable for experiments.
-  (void)l_rows; (void)r_rows; (void)groups;
-  return false;
+  // 256x256 tiles halve the bytes every CU pulls from L2 and measured faster wherever the launch
+  // still fills the GPU with them; small launches keep the 128x128 tiles (two workgroups per CU).
+  return by_default && tiles_256 >= 512;
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -484,7 +636,7 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
   AAMD_REQUIRE(lda < (1LL << 23) && K < (1LL << 23), "grouped_gemm_nt: row stride too large");
   hipStream_t st = (hipStream_t)stream;
   // tile-scaled B carries per-row R scales: use the configuration that has room for them
-  const bool large = use_large_tiles(M, N, 1);
+  const bool large = use_large_tiles(((M + 255) / 256 + (group_offsets ? E : 0)) * ((N + 255) / 256), true);
   const int BM = large ? CfgLarge::BM : CfgSmall::BM;
   const int BN = large ? (b_tile_scaled ? CfgWgrad::BN : CfgLarge::BN) : CfgSmall::BN;
   if (group_offsets) {
@@ -535,7 +687,8 @@ extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt
   p.C = dw; p.ldc = K; p.c_group_stride = expert_stride;
   p.bias = nullptr; p.bias_dtype = AAMD_NONE; p.bias_group_stride = 0;
   p.goff = group_offsets; p.tile_off = tile_ws;
-  const bool large = use_large_tiles(N, K, E);
+  // per-row scales on both operands: the 128x128 configuration measured faster for wgrad
+  const bool large = use_large_tiles(0, false);
   const int BM = large ? CfgWgrad::BM : CfgSmall::BM, BN = large ? CfgWgrad::BN : CfgSmall::BN;
   p.Lrows = N; p.Rrows = K; p.nkb = 0; p.E = E; p.nRt = (int)((K + BN - 1) / BN); p.nLt = (int)((N + BM - 1) / BM);
   p.max_kb = (int)(ld_t / kBK);
