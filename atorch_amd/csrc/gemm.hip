@@ -66,6 +66,7 @@ struct GemmParams {
   int accumulate;
   int bias_dtype;
   int gl;          // L tiles that share an R panel in the tile order
+  int ls_batch;    // kRaggedRows: L scales are fetched eight contraction blocks at a time
 };
 
 __device__ __forceinline__ v16f mfma_fp8_32x32x64(const v8i& a, const v8i& b, const v16f& c) {
@@ -135,7 +136,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   constexpr int kStage = (BM + BN) * kBK;
   constexpr int kStgBytes = 64 * 144;  // per-wave epilogue staging: 64 rows x (128 + 16) bytes
   static_assert(2 * kStage >= (NT / 64) * kStgBytes, "the epilogue staging fits in the stage buffers");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4];
+  // kRaggedRows keeps two batches of L scales besides: [BM rows][8 contraction blocks] floats each.
+  constexpr int kLsBatch = MODE == kRaggedRows ? BM * 8 * 4 : 0;
+  static_assert(NT == 2 * BM, "two threads fetch the 32 bytes of a row's scale batch");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4 + 2 * kLsBatch];
   __shared__ int slot;
   uint8_t* const Lbuf0 = lds;
   uint8_t* const Rbuf0 = lds + BM * kBK;
@@ -143,6 +147,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   uint8_t* const Rbuf1 = lds + kStage + BM * kBK;
   float* const Sc0 = reinterpret_cast<float*>(lds + 2 * kStage);
   float* const Sc1 = Sc0 + NT;
+  float* const LsB0 = Sc1 + NT;  // scale batches (kRaggedRows)
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
@@ -276,6 +281,23 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #else
   constexpr int kScaleLd = 1;
 #endif
+  // L scales of a row-major [rows, K/128] operand: one 4-byte value per row and step would touch
+  // as many cache lines as the tile itself.  Instead 32 bytes per row (eight contraction blocks)
+  // are fetched every eighth step, 16 bytes per thread, into [row][8] floats.  The last batch is
+  // shifted back so that it ends at the last block.
+  const bool batch = MODE == kRaggedRows && p.ls_batch != 0;  // uniform; implies nkb >= 8
+  const bool step_scale = !(batch && l_side);                 // this wave loads a scale every step
+  const int brow = (tid >> 1) < lvalid ? (tid >> 1) : lvalid - 1;
+  const uint32_t boff = ((uint32_t)brow * (uint32_t)p.ls_row_stride + (uint32_t)(tid & 1) * 4u) * 4u;
+  auto batch_start = [&](int b) { return 8 * b + 8 <= nkb ? 8 * b : nkb - 8; };
+  auto dma_scale_batch = [&](int b) {
+    if constexpr (MODE == kRaggedRows) {
+      const uint8_t* sb = reinterpret_cast<const uint8_t*>(Lsg + uniform_i64(l0 * p.ls_row_stride + batch_start(b)));
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   ::"v"(boff), "s"(sb), "s"(lds_addr(LsB0 + (b & 1) * (BM * 8)) + (uint32_t)(wave * 1024))
+                   : "memory");
+    }
+  };
   auto dma_scale = [&](int kb, float* Sd) {
     const uint8_t* sb = reinterpret_cast<const uint8_t*>(sbase + (int64_t)kb * s_step);
     if constexpr (kScaleLd)
@@ -283,26 +305,34 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
                    ::"v"(soff_b), "s"(sb), "s"(lds_addr(Sd) + (uint32_t)(wave * 256))
                    : "memory");
   };
-  // L half of a step: the L tile and, from the waves that own them, the L scales.
-  auto dmaL = [&](int kb, uint8_t* Ld, float* Sd) {
+  // One wave instruction of the L (R) tile of a step; the last one of a half also carries that
+  // half's scale loads.  L half: the L tile and, from the waves that own them, the L scales.
+  auto dmaL_one = [&](int n, int kb, uint8_t* Ld, float* Sd) {
     const uint8_t* lb = Lbase + (int64_t)kb * kBK;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(ltail[n] ? voffLt : voffL), "s"(lb + lslab[n]),
+                   "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
+                 : "memory");
+    if (n == C::LCH - 1 && l_side && step_scale) dma_scale(kb, Sd);
+  };
+  auto dmaR_one = [&](int n, int kb, uint8_t* Rd, float* Sd) {
+    const uint8_t* rb = Rbase + (int64_t)kb * kBK;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 ::"v"(voffR), "s"(rb + rslab[n]),
+                   "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
+                 : "memory");
+    if (n == C::RCH - 1) {
+      if (!l_side) dma_scale(kb, Sd);
+      if (batch && (kb & 7) == 0) dma_scale_batch(kb >> 3);  // lands a step before its first use
+    }
+  };
+  auto dmaL = [&](int kb, uint8_t* Ld, float* Sd) {
 #pragma unroll
-    for (int n = 0; n < C::LCH; n++)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   ::"v"(ltail[n] ? voffLt : voffL), "s"(lb + lslab[n]),
-                     "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
-                   : "memory");
-    if (l_side) dma_scale(kb, Sd);
+    for (int n = 0; n < C::LCH; n++) dmaL_one(n, kb, Ld, Sd);
   };
   auto dmaR = [&](int kb, uint8_t* Rd, float* Sd) {
-    const uint8_t* rb = Rbase + (int64_t)kb * kBK;
 #pragma unroll
-    for (int n = 0; n < C::RCH; n++)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   ::"v"(voffR), "s"(rb + rslab[n]),
-                     "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
-                   : "memory");
-    if (!l_side) dma_scale(kb, Sd);
+    for (int n = 0; n < C::RCH; n++) dmaR_one(n, kb, Rd, Sd);
   };
   auto dma = [&](int kb, uint8_t* Ld, uint8_t* Rd, float* Sd) {
     dmaL(kb, Ld, Sd);
@@ -348,9 +378,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // the workgroup barrier.  Branch free: waves outside a partial R tile compute on clamped
   // rows and skip only the final store.
   constexpr int NTILES = C::WTR * C::WTL;
-  auto compute = [&](const uint8_t* Lt, const uint8_t* Rt, const float* Sct, auto&& after_l_reads) {
+  auto compute = [&](int kb, const uint8_t* Lt, const uint8_t* Rt, const float* Sct, auto&& after_l_reads,
+                     auto&& per_tile) {
     __builtin_amdgcn_sched_barrier(0);
-    const float* Lsc = Sct;
+    // L scale of tile row r: Lsc[r * lsc_stride]
+    const int bsel = kb >> 3;
+    const float* Lsc = batch ? LsB0 + (bsel & 1) * (BM * 8) + (kb - batch_start(bsel)) : Sct;
+    const int lsc_stride = batch ? 8 : 1;
     const float* Rsc = Sct + BM;
     auto load_frag = [&](const uint8_t* T, int row, int h) {
 #if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE >= 5
@@ -368,7 +402,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       const int row = wlrow0 + j * 32 + l32;
       lf[j][0] = load_frag(Lt, row, 0);
       lf[j][1] = load_frag(Lt, row, 1);
-      cs[j] = Lsc[row] * rblk;
+      cs[j] = Lsc[row * lsc_stride] * rblk;
     }
     v8i rf[2][2];
     v4f rs[2][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
@@ -424,6 +458,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       __builtin_amdgcn_sched_barrier(0);
       // the next R row overwrites the fragment and scale slot of row i - 1, whose last fold is done
       if (j == 0 && i + 1 < C::WTR) load_r(i + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      per_tile(t);  // this sub-tile's share of the loads of the coming steps
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -446,19 +482,22 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #endif
   constexpr bool kLoads = AAMD_GEMM_ABLATE != 1 && AAMD_GEMM_ABLATE < 4, kMath = AAMD_GEMM_ABLATE < 2 || AAMD_GEMM_ABLATE >= 4;
   auto nothing = [] {};
+  auto no_feed = [](int) {};
+  // (Spreading the loads of a step over its sub-tiles instead of issuing them in one burst after
+  // the barrier measured slower: they then have less time to arrive.)
   if constexpr (!C::LAHEAD) {
     if (nkb > 0) dma(0, Lbuf0, Rbuf0, Sc0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     int kb = 0;
-    for (; kb + 1 < nkb; kb += 2) {  // two steps per trip, the stages swap roles
+    for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
       if (kLoads) dma(kb + 1, Lbuf1, Rbuf1, Sc1);
-      if (kMath) compute(Lbuf0, Rbuf0, Sc0, nothing);
+      if (kMath) compute(kb, Lbuf0, Rbuf0, Sc0, nothing, no_feed);
       dma_wait_and_sync();
       if (kLoads) dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
-      if (kMath) compute(Lbuf1, Rbuf1, Sc1, nothing);
+      if (kMath) compute(kb + 1, Lbuf1, Rbuf1, Sc1, nothing, no_feed);
       dma_wait_and_sync();
     }
-    if (kb < nkb) compute(Lbuf0, Rbuf0, Sc0, nothing);  // odd number of steps
+    if (kb < nkb) compute(kb, Lbuf0, Rbuf0, Sc0, nothing, no_feed);  // odd number of steps
   } else {
     // The L fragments of a step sit in registers for the whole step, so the L half of a stage is
     // free as soon as every wave has read it: an extra barrier after those reads lets the L tile of
@@ -467,7 +506,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     // end the loads re-read the last block to keep the counts uniform.
     auto kclamp = [&](int k) { return k < nkb ? k : nkb - 1; };
     auto wait_all_but_newest_l = [&]() {
-      if (l_side) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
+      if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
       else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
     };
     if (nkb > 0) {
@@ -475,22 +514,23 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       dmaR(0, Rbuf0, Sc0);
       dmaL(kclamp(1), Lbuf1, Sc1);
       wait_all_but_newest_l();
-      for (int kb = 0; kb < nkb; kb++) {
-        uint8_t* Lc = kb & 1 ? Lbuf1 : Lbuf0;
-        uint8_t* Rc = kb & 1 ? Rbuf1 : Rbuf0;
-        uint8_t* Rn = kb & 1 ? Rbuf0 : Rbuf1;
-        float* Sc = kb & 1 ? Sc1 : Sc0;
-        float* Sn = kb & 1 ? Sc0 : Sc1;
+      auto step = [&](int kb, uint8_t* Lc, uint8_t* Rc, float* Sc, uint8_t* Rn, float* Sn) {
         if (kLoads) dmaR(kclamp(kb + 1), Rn, Sn);
         auto mid = [&]() {
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
           if (kLoads) dmaL(kclamp(kb + 2), Lc, Sc);
         };
-        if (kMath) compute(Lc, Rc, Sc, mid);
+        if (kMath) compute(kb, Lc, Rc, Sc, mid, no_feed);
         else mid();
         if (kLoads) wait_all_but_newest_l();
         else asm volatile("s_barrier" ::: "memory");
+      };
+      int kb = 0;
+      for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
+        step(kb, Lbuf0, Rbuf0, Sc0, Rbuf1, Sc1);
+        step(kb + 1, Lbuf1, Rbuf1, Sc1, Rbuf0, Sc0);
       }
+      if (kb < nkb) step(kb, Lbuf0, Rbuf0, Sc0, Rbuf1, Sc1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
     }
   }
@@ -645,6 +685,9 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
   }
   GemmParams p = {};
   p.L = a; p.ldl = lda; p.Ls = a_s; p.ls_row_stride = K / kBK; p.ls_blk_stride = 1;
+  // 16-byte loads of scale batches need aligned rows and whole groups of four blocks
+  p.ls_batch = (K / kBK) >= 8 && (K / kBK) % 4 == 0 && (reinterpret_cast<uintptr_t>(a_s) & 15) == 0;
+  if (const char* env = getenv("AAMD_GEMM_LS_BATCH")) p.ls_batch = p.ls_batch && atoi(env) != 0;
   p.R = b; p.ldr = K; p.r_group_stride = N * K;
   p.Rs = b_s;
   p.rs_row_stride = K / kBK; p.rs_blk_stride = 1;
