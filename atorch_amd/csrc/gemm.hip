@@ -176,7 +176,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     const int in_grp = (int)(pid % width);
     lt = first + in_grp % gsz;
     rt = in_grp / gsz;
-#if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE == 3
+#if defined(AAMD_GEMM_ABLATE) && (AAMD_GEMM_ABLATE == 3 || AAMD_GEMM_HOT)
     lt = 0; rt = 0;  // measurement build: every workgroup streams the same tile
 #endif
   }
@@ -422,9 +422,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     constexpr int D = PRB - 1;
     v16f pr[PRB];
     load_r(0);
-    __builtin_amdgcn_sched_barrier(0);
-    after_l_reads();  // the L fragments and L scales of this step are on their way to registers
-    __builtin_amdgcn_sched_barrier(0);
     // acc of sub-tile t += raw product * scales, registers [8*half, 8*half + 8) of the sub-tile
     auto fold_half = [&](int t, int half) {
       const int i = t / C::WTL, j = t % C::WTL;
@@ -459,7 +456,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       // the next R row overwrites the fragment and scale slot of row i - 1, whose last fold is done
       if (j == 0 && i + 1 < C::WTR) load_r(i + 1);
       __builtin_amdgcn_sched_barrier(0);
-      per_tile(t);  // this sub-tile's share of the loads of the coming steps
+      // every L fragment has been an MFMA operand by now, so it has left the LDS: the hook (a
+      // barrier and the next L loads) costs no extra wait here
+      if (t == C::WTL - 1) after_l_reads();
+      per_tile(t);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -479,6 +479,9 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // work, to time the two halves of the pipeline separately.  Results are wrong in both.
 #ifndef AAMD_GEMM_ABLATE
 #define AAMD_GEMM_ABLATE 0
+#endif
+#ifndef AAMD_GEMM_HOT
+#define AAMD_GEMM_HOT 0
 #endif
   constexpr bool kLoads = AAMD_GEMM_ABLATE != 1 && AAMD_GEMM_ABLATE < 4, kMath = AAMD_GEMM_ABLATE < 2 || AAMD_GEMM_ABLATE >= 4;
   auto nothing = [] {};
