@@ -48,6 +48,8 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
                                                           const int32_t* __restrict__ row_map, int topk,
                                                           int64_t M_out, uint8_t* __restrict__ q,
                                                           float* __restrict__ s, float eps) {
+  // the three-instruction division is checked for bf16 values over scales of bf16 maxima only
+  const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
   const int64_t base = (int64_t)blockIdx.x * (16 * U);
   const int64_t cols = (int64_t)nt * kTile;
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     float v[8];
     raw[u].get(v);
     const float sc = scale_from_amax(row16_max(amax8(v)), eps);
-    const v2i codes = quant8(v, sc);
+    const v2i codes = quant8(v, sc, plain_div);
     if (!valid[u]) continue;
     if constexpr (!SCATTER) {
       *reinterpret_cast<v2i*>(q + row[u] * cols + (int64_t)tc[u] * kTile + l * 8) = codes;
@@ -112,14 +114,14 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
 // codes of the 8x8 register block, transposed through LDS, written as rows of 128 bytes:
 // out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
 __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const float* cs, uint8_t* tile_t,
-                                                 uint8_t* __restrict__ out, int64_t ld_out) {
+                                                 uint8_t* __restrict__ out, int64_t ld_out, bool plain_div) {
   const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
     float col[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) col[i] = v[i][j];
-    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cs[j]);
+    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cs[j], plain_div);
   }
   __syncthreads();
 #pragma unroll
@@ -136,6 +138,7 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps) {
+  const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
   __shared__ float part[16][kTile];
   __shared__ float cscale[kTile];
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     if (q != nullptr) {
       const float sc = scale_from_amax(row16_max(amax8(v[i])), eps);
       const int r = gr * 8 + i;
-      const v2i codes = quant8(v[i], sc);
+      const v2i codes = quant8(v[i], sc, plain_div);
       if (r < mvalid) {
         *reinterpret_cast<v2i*>(q + (m0 + r) * cols + (int64_t)kc * kTile + c * 8) = codes;
         if (c == 0) s[(m0 + r) * nt + kc] = sc;
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   float cs[8];
 #pragma unroll
   for (int j = 0; j < 8; j++) cs[j] = cscale[c * 8 + j];
-  store_transposed(v, cs, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
+  store_transposed(v, cs, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t, plain_div);
 }
 
 template <typename IN>
@@ -196,6 +199,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
                                                             uint8_t* __restrict__ q, float* __restrict__ s,
                                                             uint8_t* __restrict__ q_t, float* __restrict__ s_t,
                                                             float eps) {
+  const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
   __shared__ float part[16];
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
   const int kb = blockIdx.x, nb = blockIdx.y, e = blockIdx.z;
@@ -220,12 +224,12 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
   uint8_t* qe = q + (int64_t)e * N * K + (int64_t)nb * kTile * K + (int64_t)kb * kTile;
 #pragma unroll
   for (int i = 0; i < 8; i++)
-    *reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8) = quant8(v[i], sc);
+    *reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8) = quant8(v[i], sc, plain_div);
   if (q_t != nullptr) {
     float cs[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) cs[j] = sc;
-    store_transposed(v, cs, tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, N);
+    store_transposed(v, cs, tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, N, plain_div);
   }
 }
 

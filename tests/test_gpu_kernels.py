@@ -14,6 +14,10 @@ GEMM_TOL = 1e-2  # bf16 output, the tolerance the path is specified to
 GEMM_TOL_F32 = 5e-4
 
 
+def _u8q(t):
+    return t.view(torch.uint8)
+
+
 def _u8(t):
     return t.view(torch.uint8).cpu()
 
@@ -53,6 +57,42 @@ def test_tile_quant_all_bf16_patterns(oracle, dev):
     qo, so = oracle.tile_quant(x)
     assert torch.equal(s.cpu(), so)
     assert torch.equal(_u8(q), qo)
+
+
+def test_tile_quant_division_is_exact_over_the_whole_bf16_domain(oracle, dev):
+    """The kernels divide by a tile's scale with a hoisted reciprocal and an FMA correction instead
+    of one IEEE division per element.  Every pair (x, amax) of finite bf16 values with |x| <= amax
+    (about 10^9 quotients) must give the code of the IEEE quotient fl(x / fl(amax / 448)); the
+    reference is torch's own fp32 division and fp8 cast on the device, itself compared with the
+    CPU oracle on a sample of the same tiles."""
+    from atorch_amd import kernels
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = bits[torch.isfinite(bits.float())]
+    pad = (-finite.numel()) % (TILE - 1)
+    vals = torch.cat([finite, torch.zeros(pad, dtype=torch.bfloat16)]).view(-1, TILE - 1).to(dev)  # [515, 127]
+    amaxes = finite[finite.float() > 0].to(dev)  # every positive finite bf16 value, subnormals included
+    absvals = vals.float().abs()
+    chunk = 64
+    bad = 0
+    for lo in range(0, amaxes.numel(), chunk):
+        a = amaxes[lo : lo + chunk]  # [c]
+        keep = absvals.unsqueeze(0) <= a.float().view(-1, 1, 1)
+        body = torch.where(keep, vals.unsqueeze(0), torch.zeros((), dtype=torch.bfloat16, device=dev))
+        first = a.view(-1, 1, 1).expand(-1, vals.shape[0], 1)
+        x = torch.cat([first, body], dim=2).reshape(-1, TILE).contiguous()
+        q, s = kernels.tile_quant(x)
+        s_ref = (a.float().cpu() / torch.full((a.numel(),), 448.0)).to(dev)  # IEEE division on the host
+        s_ref = s_ref.view(-1, 1).expand(-1, vals.shape[0]).reshape(-1, 1)
+        assert torch.equal(s, s_ref)
+        q_ref = (x.float() / s_ref).to(torch.float8_e4m3fn)
+        neq = _u8q(q) != _u8q(q_ref)
+        bad += int(neq.sum())
+        if lo % (chunk * 64) == 0:  # the device-side reference against the oracle
+            rows = torch.arange(0, x.shape[0], 97, device=dev)
+            qo, so = oracle.tile_quant(x[rows].cpu())
+            assert torch.equal(_u8q(q_ref[rows]).cpu(), qo) and torch.equal(s[rows].cpu(), so)
+    assert bad == 0, f"{bad} quotients differ from the IEEE division"
 
 
 def test_tile_quant_known_answers(dev):
