@@ -37,13 +37,14 @@ int hip_fail(hipError_t e, const char* what);
 // ---- scalar conversions ---------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// fp32 -> bf16 bits, round to nearest even (finite inputs and inf; NaN stays NaN).
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+// fp32 -> bf16 bits, round to nearest even: gfx950 has the conversion in hardware
+// (v_cvt_pk_bf16_f32, two values per instruction).
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
 
 // Input element loaders: 8 consecutive elements -> 8 floats.
 struct BF16 {

@@ -87,8 +87,8 @@ __device__ __forceinline__ void store4(OUT* dst, v4f o, bool accumulate) {
       o[3] += bf16_bits_to_f32((uint32_t)old[1] >> 16);
     }
     v2i w;
-    w[0] = (int)(f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16));
-    w[1] = (int)(f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16));
+    w[0] = (int)pack_bf16x2(o[0], o[1]);
+    w[1] = (int)pack_bf16x2(o[2], o[3]);
     *reinterpret_cast<v2i*>(dst) = w;
   }
 }
@@ -584,8 +584,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
               *reinterpret_cast<v4f*>(dst) = o;
             } else {
               v2i w;
-              w[0] = (int)(f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16));
-              w[1] = (int)(f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16));
+              w[0] = (int)pack_bf16x2(o[0], o[1]);
+              w[1] = (int)pack_bf16x2(o[2], o[3]);
               *reinterpret_cast<v2i*>(dst) = w;
             }
           }

@@ -32,25 +32,41 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
   }
   __syncthreads();
   const int64_t H = (int64_t)H8 * 8;
-  for (int c = threadIdx.x; c < H8; c += 256) {
+  for (int c = threadIdx.x; c < H8; c += blockDim.x) {
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
-#pragma unroll 4
+#ifndef AAMD_UNP_UNROLL
+#define AAMD_UNP_UNROLL 4
+#endif
+#ifndef AAMD_UNP_NT
+#define AAMD_UNP_NT 1
+#endif
+#pragma unroll AAMD_UNP_UNROLL
     for (int j = 0; j < topk; j++) {
       const int r = srow[j];
       if (r < 0) continue;
-      const v4i raw = *reinterpret_cast<const v4i*>(y + (int64_t)r * H + c * 8);
+      const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)r * H + c * 8);
+      const v4i raw = AAMD_UNP_NT ? __builtin_nontemporal_load(src) : *src;
       float v[8];
       unpack8(raw, v);
       const float pv = sprob[j];
+      // separate multiply and add (no FMA contraction): the reference multiplies, rounds the
+      // product to the promoted dtype, then sums
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        float prod = v[i];
-        // separate multiply and add (no FMA contraction): the reference multiplies, rounds, then sums
-        if constexpr (PD == AAMD_BF16) prod = bf16_bits_to_f32(f32_to_bf16_bits((v[i] * pv)));
-        if constexpr (PD == AAMD_F32) prod = (v[i] * pv);
-        acc[i] = acc[i] + prod;
+      for (int i = 0; i < 8; i += 2) {
+        float p0 = v[i], p1 = v[i + 1];
+        if constexpr (PD == AAMD_BF16) {
+          const uint32_t pk = pack_bf16x2(v[i] * pv, v[i + 1] * pv);
+          p0 = __uint_as_float(pk << 16);
+          p1 = __uint_as_float(pk & 0xffff0000u);
+        }
+        if constexpr (PD == AAMD_F32) {
+          p0 = v[i] * pv;
+          p1 = v[i + 1] * pv;
+        }
+        acc[i] = acc[i] + p0;
+        acc[i + 1] = acc[i + 1] + p1;
       }
     }
     if constexpr (PD == AAMD_F32) {
@@ -60,7 +76,7 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
     } else {
       v4i w;
 #pragma unroll
-      for (int i = 0; i < 4; i++) w[i] = (int)(f32_to_bf16_bits(acc[2 * i]) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16));
+      for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
       *reinterpret_cast<v4i*>(reinterpret_cast<u16*>(out) + t * H + c * 8) = w;
     }
   }

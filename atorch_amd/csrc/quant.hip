@@ -74,14 +74,22 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     const float sc = scale_from_amax(row16_max(amax8(v)), eps);
     const v2i codes = quant8(v, sc, plain_div);
     if (!valid[u]) continue;
+#ifndef AAMD_QUANT_NT_STORE
+#define AAMD_QUANT_NT_STORE 1
+#endif
+    auto put = [&](v2i* dst, v2i val) {
+      // the codes are not read again by this kernel: streaming stores keep them out of the way
+      if (AAMD_QUANT_NT_STORE) __builtin_nontemporal_store(val, dst);
+      else *dst = val;
+    };
     if constexpr (!SCATTER) {
-      *reinterpret_cast<v2i*>(q + row[u] * cols + (int64_t)tc[u] * kTile + l * 8) = codes;
+      put(reinterpret_cast<v2i*>(q + row[u] * cols + (int64_t)tc[u] * kTile + l * 8), codes);
       if (l == 0) s[row[u] * nt + tc[u]] = sc;
     } else {
       for (int j = 0; j < topk; j++) {
         const int64_t dst = row_map[row[u] * topk + j];
         if (dst < 0 || dst >= M_out) continue;
-        *reinterpret_cast<v2i*>(q + dst * cols + (int64_t)tc[u] * kTile + l * 8) = codes;
+        put(reinterpret_cast<v2i*>(q + dst * cols + (int64_t)tc[u] * kTile + l * 8), codes);
         if (l == 0) s[dst * nt + tc[u]] = sc;
       }
     }
@@ -293,8 +301,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
     v4i w0, w1;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      w0[i] = (int)(f32_to_bf16_bits(o[2 * i]) | (f32_to_bf16_bits(o[2 * i + 1]) << 16));
-      w1[i] = (int)(f32_to_bf16_bits(o[8 + 2 * i]) | (f32_to_bf16_bits(o[8 + 2 * i + 1]) << 16));
+      w0[i] = (int)pack_bf16x2(o[2 * i], o[2 * i + 1]);
+      w1[i] = (int)pack_bf16x2(o[8 + 2 * i], o[8 + 2 * i + 1]);
     }
     reinterpret_cast<v4i*>(dst)[0] = w0;
     reinterpret_cast<v4i*>(dst)[1] = w1;
@@ -334,7 +342,10 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   const int64_t total = T * nt;
   AAMD_REQUIRE(total < (int64_t)1 << 40, "quant_1x128: too many tiles");
   hipStream_t st = (hipStream_t)stream;
-  constexpr int U = 4;
+#ifndef AAMD_QUANT_U
+#define AAMD_QUANT_U 2
+#endif
+  constexpr int U = AAMD_QUANT_U;
   const int64_t blocks = (total + 16 * U - 1) / (16 * U);
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "quant_1x128: grid too large");
   dim3 grid((unsigned)blocks), block(256);
