@@ -150,6 +150,14 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   float* const LsB0 = Sc1 + NT;  // scale batches (kRaggedRows)
 
   const int tid = threadIdx.x;
+#ifdef AAMD_GEMM_TIMING
+  // measurement build: six time stamps per workgroup go where the bias would be read from
+  unsigned long long stamp[6];
+  stamp[0] = __builtin_readcyclecounter();
+#define AAMD_STAMP(i) stamp[i] = __builtin_readcyclecounter()
+#else
+#define AAMD_STAMP(i)
+#endif
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
   const int lane = tid & 63;
 
@@ -210,6 +218,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     if (kb0 + nkb > p.max_kb) nkb = p.max_kb > kb0 ? p.max_kb - kb0 : 0;  // never read past the buffers
   }
   g = __builtin_amdgcn_readfirstlane(g);
+  AAMD_STAMP(1);
   const int64_t r0 = (int64_t)rt * BN;
   const int64_t rleft = p.Rrows - r0;
   const int rvalid = rleft < BN ? (int)rleft : BN;  // a multiple of 128
@@ -516,7 +525,9 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       dmaL(0, Lbuf0, Sc0);
       dmaR(0, Rbuf0, Sc0);
       dmaL(kclamp(1), Lbuf1, Sc1);
+      AAMD_STAMP(2);
       wait_all_but_newest_l();
+      AAMD_STAMP(3);
       auto step = [&](int kb, uint8_t* Lc, uint8_t* Rc, float* Sc, uint8_t* Rn, float* Sn) {
         if (kLoads) dmaR(kclamp(kb + 1), Rn, Sn);
         auto mid = [&]() {
@@ -543,12 +554,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // would be 8-byte pieces in 32 different rows per instruction.  Each wave instead transposes its
   // tile through its own LDS region and writes 128-byte row segments: 8 lanes x 16 bytes per row.
   if (MODE == kRaggedK && nkb == 0 && p.accumulate) return;  // empty group: leave dW untouched
+  AAMD_STAMP(4);
   __syncthreads();  // every wave is done with the stage buffers
   if (!wave_active) return;
   OUT* Cg = reinterpret_cast<OUT*>(p.C) + (int64_t)g * p.c_group_stride;
   uint8_t* const stg = lds + wave * kStgBytes;
   constexpr int WROWS = C::WTL * 32;
-  static_assert(WROWS == 64, "the staging region holds 64 rows");
+  static_assert(WROWS <= 64 && WROWS % 8 == 0, "the staging region holds 64 rows");
   auto flush = [&](auto tag) {
     using ST = decltype(tag);  // staging type: OUT, or float when the old output is added in fp32
     constexpr int CW = 128 / (int)sizeof(ST);  // columns per chunk
@@ -565,7 +577,11 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
         for (int q = 0; q < 4; q++) {
           const int64_t rcol = r0 + wrow0 + i * 32 + 8 * q + 4 * hg;
           v4f b4 = {0.f, 0.f, 0.f, 0.f};
+#ifdef AAMD_GEMM_TIMING
+          if (false) {
+#else
           if (MODE == kRaggedRows && p.bias != nullptr) {
+#endif
             if (p.bias_dtype == AAMD_F32) {
               b4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(p.bias) + g * p.bias_group_stride + rcol);
             } else {
@@ -622,6 +638,15 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     if (p.accumulate) flush(float{});
     else flush(u16{});
   }
+#ifdef AAMD_GEMM_TIMING
+  stamp[1] = __builtin_readcyclecounter();  // epilogue issued (overwrites the group-lookup stamp)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  stamp[5] = __builtin_readcyclecounter();
+  if (tid == 0 && p.bias != nullptr) {
+    unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 6;
+    for (int i = 0; i < 6; i++) dst[i] = stamp[i];
+  }
+#endif
 }
 
 int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st);
