@@ -17,7 +17,7 @@ struct Raw8;
 template <>
 struct Raw8<BF16> {
   v4i a;
-  __device__ __forceinline__ void load(const u16* p) { a = *reinterpret_cast<const v4i*>(p); }
+  __device__ __forceinline__ void load(const u16* p) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const { unpack8(a, v); }
 };
@@ -25,8 +25,8 @@ template <>
 struct Raw8<F32> {
   v4i a, b;
   __device__ __forceinline__ void load(const float* p) {
-    a = reinterpret_cast<const v4i*>(p)[0];
-    b = reinterpret_cast<const v4i*>(p)[1];
+    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+    b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p) + 1);
   }
   __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const {
@@ -136,8 +136,8 @@ __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const f
   for (int n = 0; n < 4; n++) {
     const int idx = threadIdx.x + 256 * n;
     const int r = idx >> 3, ch = idx & 7;
-    *reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16) =
-        *reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16);
+    __builtin_nontemporal_store(*reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16),
+                                reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16));
   }
 }
 
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
       const int r = gr * 8 + i;
       const v2i codes = quant8(v[i], sc, plain_div);
       if (r < mvalid) {
-        *reinterpret_cast<v2i*>(q + (m0 + r) * cols + (int64_t)kc * kTile + c * 8) = codes;
+        __builtin_nontemporal_store(codes, reinterpret_cast<v2i*>(q + (m0 + r) * cols + (int64_t)kc * kTile + c * 8));
         if (c == 0) s[(m0 + r) * nt + kc] = sc;
       }
     }
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
   uint8_t* qe = q + (int64_t)e * N * K + (int64_t)nb * kTile * K + (int64_t)kb * kTile;
 #pragma unroll
   for (int i = 0; i < 8; i++)
-    *reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8) = quant8(v[i], sc, plain_div);
+    __builtin_nontemporal_store(quant8(v[i], sc, plain_div), reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8));
   if (q_t != nullptr) {
     float cs[8];
 #pragma unroll
