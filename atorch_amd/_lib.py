@@ -30,6 +30,11 @@ SIGNATURES = {
         _int,
         [_vp, _int, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _f32, _vp],
     ),
+    "aamd_swiglu_quant_1x128": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "aamd_swiglu_quant_1x128_dual_grouped": (
+        _int,
+        [_vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+    ),
     "aamd_quant_128x128": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp]),
     "aamd_dequant": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _int, _vp]),
     "aamd_grouped_gemm_fp8_nt": (

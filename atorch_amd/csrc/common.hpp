@@ -50,6 +50,11 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16
 struct BF16 {
   typedef u16 elem;
 };
+// bf16 rows [a | b] of a gated linear unit: the element read at column c is
+// h = bf16(bf16(silu(a[c])) * b[c]) with b = a + gate_off (grouped_gemm_moe.py:331-334).
+struct GLU {
+  typedef u16 elem;
+};
 struct F32 {
   typedef float elem;
 };

@@ -17,14 +17,14 @@ struct Raw8;
 template <>
 struct Raw8<BF16> {
   v4i a;
-  __device__ __forceinline__ void load(const u16* p) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
+  __device__ __forceinline__ void load(const u16* p, int64_t) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const { unpack8(a, v); }
 };
 template <>
 struct Raw8<F32> {
   v4i a, b;
-  __device__ __forceinline__ void load(const float* p) {
+  __device__ __forceinline__ void load(const float* p, int64_t) {
     a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
     b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p) + 1);
   }
@@ -38,6 +38,41 @@ struct Raw8<F32> {
   }
 };
 
+// SwiGLU on load: a and b halves of a row, h = silu(a) * b with both roundings to bf16 that the
+// reference's two torch ops make (F.silu on a bf16 tensor, then the product; fp32 inside).
+template <>
+struct Raw8<GLU> {
+  v4i a, b;
+  __device__ __forceinline__ void load(const u16* p, int64_t gate_off) {
+    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+    b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p + gate_off));
+  }
+  __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v) const {
+    float fa[8], fb[8];
+    unpack8(a, fa);
+    unpack8(b, fb);
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      // hardware exp2 and reciprocal: a few fp32 ulps, far below the bf16 rounding that follows
+      const float s0 = __fdividef(fa[i], 1.0f + __expf(-fa[i]));
+      const float s1 = __fdividef(fa[i + 1], 1.0f + __expf(-fa[i + 1]));
+      const uint32_t sl = pack_bf16x2(s0, s1);
+      const uint32_t h = pack_bf16x2(__uint_as_float(sl << 16) * fb[i], __uint_as_float(sl & 0xffff0000u) * fb[i + 1]);
+      v[i] = __uint_as_float(h << 16);
+      v[i + 1] = __uint_as_float(h & 0xffff0000u);
+    }
+  }
+};
+
+// 8 values that are bf16-representable -> 16 bytes
+__device__ __forceinline__ v4i pack8_bf16(const float* v) {
+  v4i w;
+#pragma unroll
+  for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(v[2 * i], v[2 * i + 1]);
+  return w;
+}
+
 // ---------------------------------------------------------------------------------------
 // 1x128 quant, 16 lanes per tile, U tiles per lane group.  SCATTER: write each quantised
 // row to its topk destinations (row_map), reading it once.
@@ -47,7 +82,8 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
                                                           int nt, int64_t total_tiles,
                                                           const int32_t* __restrict__ row_map, int topk,
                                                           int64_t M_out, uint8_t* __restrict__ q,
-                                                          float* __restrict__ s, float eps) {
+                                                          float* __restrict__ s, float eps, int64_t gate_off,
+                                                          u16* __restrict__ h_out) {
   // the three-instruction division is checked for bf16 values over scales of bf16 maxima only
   const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
@@ -65,7 +101,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     if (!valid[u]) tile = total_tiles - 1;
     row[u] = tile / nt;
     tc[u] = (int)(tile - row[u] * nt);
-    raw[u].load(x + row[u] * ldx + (int64_t)tc[u] * kTile + l * 8);
+    raw[u].load(x + row[u] * ldx + (int64_t)tc[u] * kTile + l * 8, gate_off);
   }
 #pragma unroll
   for (int u = 0; u < U; u++) {
@@ -74,6 +110,8 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     const float sc = scale_from_amax(row16_max(amax8(v)), eps);
     const v2i codes = quant8(v, sc, plain_div);
     if (!valid[u]) continue;
+    if (h_out != nullptr)  // the gated activation itself, for callers that keep it
+      *reinterpret_cast<v4i*>(h_out + row[u] * cols + (int64_t)tc[u] * kTile + l * 8) = pack8_bf16(v);
 #ifndef AAMD_QUANT_NT_STORE
 #define AAMD_QUANT_NT_STORE 1
 #endif
@@ -104,14 +142,14 @@ constexpr int kTLd = kTile + 16;  // LDS row stride (bytes) of the transposed co
 
 template <typename IN>
 __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, int64_t ldx, int rows_valid,
-                                          float (&v)[8][8]) {
+                                          float (&v)[8][8], int64_t gate_off = 0) {
   const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
   Raw8<IN> raw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const int r = gr * 8 + i;
     if (r < rows_valid)
-      raw[i].load(x + (int64_t)r * ldx + c * 8);
+      raw[i].load(x + (int64_t)r * ldx + c * 8, gate_off);
     else
       raw[i].zero();
   }
@@ -145,7 +183,8 @@ template <typename IN>
 __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
-    uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps) {
+    uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
+    u16* __restrict__ h_out) {
   const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
   __shared__ float part[16][kTile];
   __shared__ float cscale[kTile];
@@ -162,7 +201,7 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
 
   float v[8][8];
-  load_tile<IN>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v);
+  load_tile<IN>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
 
   // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
   float cm[8];
@@ -172,6 +211,8 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   for (int i = 0; i < 8; i++) {
 #pragma unroll
     for (int j = 0; j < 8; j++) cm[j] = fmaxf(cm[j], fabsf(v[i][j]));
+    if (h_out != nullptr && gr * 8 + i < mvalid)
+      *reinterpret_cast<v4i*>(h_out + (m0 + gr * 8 + i) * cols + (int64_t)kc * kTile + c * 8) = pack8_bf16(v[i]);
     if (q != nullptr) {
       const float sc = scale_from_amax(row16_max(amax8(v[i])), eps);
       const int r = gr * 8 + i;
@@ -351,14 +392,14 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   dim3 grid((unsigned)blocks), block(256);
   if (row_map == nullptr) {
     if (x_dtype == AAMD_BF16)
-      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps);
+      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
     else
-      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps);
+      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
   } else {
     if (x_dtype == AAMD_BF16)
-      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps);
+      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
     else
-      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps);
+      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
   }
   AAMD_LAUNCH_CHECK("quant_1x128");
   return AAMD_OK;
@@ -391,10 +432,59 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
   dim3 grid((unsigned)(cols / kTile), (unsigned)grid_tiles), block(256);
   const int nt = (int)(cols / kTile);
   if (x_dtype == AAMD_BF16)
-    quant_dual_grouped_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+    quant_dual_grouped_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
   else
-    quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+    quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
   AAMD_LAUNCH_CHECK("quant_dual_grouped");
+  return AAMD_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// SwiGLU fused into the quantisation of the intermediate activations
+// ---------------------------------------------------------------------------------------
+extern "C" int aamd_swiglu_quant_1x128(const void* fc1, int64_t rows, int64_t F, int64_t ld, void* h_out, uint8_t* q,
+                                       float* s, void* stream) {
+  AAMD_REQUIRE(rows >= 0 && F >= 0 && F % kTile == 0, "swiglu_quant: F=%lld must be a multiple of 128", (long long)F);
+  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0, "swiglu_quant: ld=%lld must be >= 2F and a multiple of 8", (long long)ld);
+  if (rows == 0 || F == 0) return AAMD_OK;
+  AAMD_REQUIRE(fc1 && q && s, "swiglu_quant: null pointer");
+  AAMD_REQUIRE(aligned16(fc1) && aligned16(q) && aligned16(h_out), "swiglu_quant: pointers must be 16-byte aligned");
+  const int nt = (int)(F / kTile);
+  const int64_t total = rows * nt;
+  AAMD_REQUIRE(total < (int64_t)1 << 40, "swiglu_quant: too many tiles");
+  constexpr int U = AAMD_QUANT_U;
+  const int64_t blocks = (total + 16 * U - 1) / (16 * U);
+  AAMD_REQUIRE(blocks < 0x7fffffffLL, "swiglu_quant: grid too large");
+  quant_1x128_kernel<GLU, false, U><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+      (const u16*)fc1, ld, nt, total, nullptr, 1, rows, q, s, 0.f, F, (u16*)h_out);
+  AAMD_LAUNCH_CHECK("swiglu_quant_1x128");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, int64_t F, int64_t ld,
+                                                    const int64_t* group_offsets, int E, int32_t* tile_ws,
+                                                    void* h_out, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
+                                                    int64_t ld_t, void* stream) {
+  AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "swiglu_quant_dual: F=%lld must be a multiple of 128", (long long)F);
+  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0, "swiglu_quant_dual: bad ld=%lld", (long long)ld);
+  AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "swiglu_quant_dual: group_offsets / tile_ws required");
+  AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "swiglu_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
+  AAMD_REQUIRE((q == nullptr) == (s == nullptr), "swiglu_quant_dual: q and s go together");
+  AAMD_REQUIRE(q_t && s_t, "swiglu_quant_dual: q_t / s_t required");
+  if (F == 0) return AAMD_OK;
+  const int64_t max_tiles = M / kTile + E;
+  const int64_t grid_tiles = ld_t / kTile < max_tiles ? ld_t / kTile : max_tiles;
+  if (grid_tiles == 0) return AAMD_OK;
+  AAMD_REQUIRE(aligned16(fc1) && aligned16(q_t) && (!q || aligned16(q)) && aligned16(h_out),
+               "swiglu_quant_dual: pointers must be 16-byte aligned");
+  AAMD_REQUIRE(grid_tiles <= 65535, "swiglu_quant_dual: more than 65535 token tiles");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
+  if (rc) return rc;
+  dim3 grid((unsigned)(F / kTile), (unsigned)grid_tiles), block(256);
+  quant_dual_grouped_kernel<GLU><<<grid, block, 0, st>>>((const u16*)fc1, ld, (int)(F / kTile), group_offsets, tile_ws, E,
+                                                         q, s, q_t, s_t, ld_t, 0.f, F, (u16*)h_out);
+  AAMD_LAUNCH_CHECK("swiglu_quant_dual_grouped");
   return AAMD_OK;
 }
 

@@ -198,6 +198,57 @@ def tile_quant_dual_grouped(
     return q, s, q_t, s_t
 
 
+def swiglu_tile_quant(fc1: torch.Tensor, return_activation: bool = False):
+    """``h = silu(fc1[..., :F]) * fc1[..., F:]`` (SwiGLUActivatition, grouped_gemm_moe.py:331-334)
+    quantised 1x128 along the last dim without writing ``h``.  Returns ``(q, s)`` or
+    ``(q, s, h)`` (``h`` bf16) with ``return_activation``."""
+    assert fc1.dtype == torch.bfloat16 and fc1.stride(-1) == 1 and fc1.is_contiguous()
+    two_f = fc1.size(-1)
+    assert two_f % (2 * TILE) == 0, "the gated width must be a multiple of 128"
+    F = two_f // 2
+    rows = fc1.numel() // two_f if two_f else 0
+    dev = fc1.device
+    q = torch.empty(*fc1.shape[:-1], F, dtype=FP8, device=dev)
+    s = torch.empty(*fc1.shape[:-1], F // TILE, dtype=torch.float32, device=dev)
+    h = torch.empty(*fc1.shape[:-1], F, dtype=torch.bfloat16, device=dev) if return_activation else None
+    check(lib().aamd_swiglu_quant_1x128(ptr(fc1), rows, F, two_f, ptr(h), ptr(q), ptr(s), stream()))
+    return (q, s, h) if return_activation else (q, s)
+
+
+def swiglu_tile_quant_dual_grouped(
+    fc1: torch.Tensor,
+    group_offsets: torch.Tensor,
+    num_groups: int,
+    ld_t: Optional[int] = None,
+    rowwise: bool = True,
+    return_activation: bool = False,
+):
+    """SwiGLU fused into ``tile_quant_dual_grouped``: row-wise and transposed 1x128 quantisation of
+    ``h = silu(a) * b`` for rows ``[a | b]`` of ``fc1 [M, 2F]``.  Returns ``(q, s, q_t, s_t)`` (plus
+    ``h`` with ``return_activation``), layouts as ``tile_quant_dual_grouped``."""
+    assert fc1.dim() == 2 and fc1.is_contiguous() and fc1.dtype == torch.bfloat16
+    M, two_f = fc1.shape
+    assert two_f % (2 * TILE) == 0
+    F = two_f // 2
+    assert group_offsets.dtype == torch.int64 and group_offsets.numel() == num_groups + 1
+    if ld_t is None:
+        ld_t = padded_bound(M, num_groups)
+    dev = fc1.device
+    q = torch.empty((M, F), dtype=FP8, device=dev) if rowwise else None
+    s = torch.empty((M, F // TILE), dtype=torch.float32, device=dev) if rowwise else None
+    q_t = torch.empty((F, ld_t), dtype=FP8, device=dev)
+    s_t = torch.empty((ld_t // TILE, F), dtype=torch.float32, device=dev)
+    h = torch.empty((M, F), dtype=torch.bfloat16, device=dev) if return_activation else None
+    ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
+    check(
+        lib().aamd_swiglu_quant_1x128_dual_grouped(
+            ptr(fc1), M, F, two_f, ptr(group_offsets), num_groups, ptr(ws), ptr(h),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, stream(),
+        )
+    )  # fmt: skip
+    return (q, s, q_t, s_t, h) if return_activation else (q, s, q_t, s_t)
+
+
 def block_quant_batched(w: torch.Tensor, eps: float = 0.0, return_transpose: bool = False):
     """128x128 block quantisation of ``w [E, N, K]`` in one launch.
     Returns ``(q [E,N,K], s [E,N/128,K/128], q_t [E,K,N] | None, s_t [E,K/128,N/128] | None)``."""

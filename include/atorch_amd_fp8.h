@@ -111,6 +111,26 @@ int aamd_dequant(const uint8_t *q, const float *s, int64_t M, int64_t N, int til
                  void *stream);
 
 /*
+ * SwiGLU fused into the 1x128 quantisation of the intermediate activations (the step between
+ * the two grouped GEMMs of an expert MLP): for rows [a | b] of the first GEMM's output,
+ *   h = bf16(bf16(silu(a)) * b)   (silu(x) = x / (1 + exp(-x)) in fp32)
+ * is quantised like aamd_quant_1x128 / aamd_quant_1x128_dual_grouped would quantise h, without h
+ * making a round trip through memory.
+ * Replaces SwiGLUActivatition.forward, atorch/modules/moe/grouped_gemm_moe.py:331-334 (torch.chunk,
+ * F.silu, multiply), as used between the gmm calls of compute_moe, :845-850, followed by the
+ * per-expert quantize_op.quantize of the next grouped linear, quantized_grouped_linear.py:90-101.
+ *   fc1 [rows, 2F] bf16 (row stride ld elements, ld >= 2F), F % 128 == 0
+ *   h_out [rows, F] bf16 or NULL (the activation itself, for callers that keep it)
+ *   q [rows, F], s [rows, F/128]; the dual form adds q_t / s_t with the layouts, scratch and
+ *   group_offsets of aamd_quant_1x128_dual_grouped (q and s may then be NULL).
+ */
+int aamd_swiglu_quant_1x128(const void *fc1, int64_t rows, int64_t F, int64_t ld, void *h_out, uint8_t *q, float *s,
+                            void *stream);
+int aamd_swiglu_quant_1x128_dual_grouped(const void *fc1, int64_t M, int64_t F, int64_t ld,
+                                         const int64_t *group_offsets, int E, int32_t *tile_ws, void *h_out,
+                                         uint8_t *q, float *s, uint8_t *q_t, float *s_t, int64_t ld_t, void *stream);
+
+/*
  * Ragged grouped block-scaled GEMM, "NT": for every group g and its rows m,
  *   C[m, n] = sum_kb dot(A[m, kb], B_g[n, kb]) * a_s[m, kb] * b_s_g[n/128 or n, kb]  (+ bias_g[n])
  * fp8 x fp8 MFMA, fp32 accumulation, scales applied per 128-deep block.

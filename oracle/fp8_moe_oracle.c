@@ -26,6 +26,9 @@
  *       pure-Python brute force in the reference's accumulation order, linearity / accumulate,
  *       grouped == per-expert loop, fp64 autograd of the unquantised problem (roles and transposes)
  *   oracle_permute_indices                        pinned: torch.argsort(stable=True), bincount
+ *   oracle_swiglu_bf16                            pinned: torch's CPU F.silu and multiply on bf16 tensors
+ *       (equal except where fp32 silu rounds differently: at most one bf16 ulp, counted in the test),
+ *       closed forms silu(0) = 0, silu(x) -> x and -> -0 for large |x|, h == b * silu(a) in double
  *   oracle_unpermute_combine                      pinned: brute force, torch restatement (index_copy_,
  *       multiply, sum) bit-exact for bf16 weights, inverse-of-permute property
  * Parity unpinned (nothing available here can pin it; the oracle's choice is stated instead):
@@ -334,5 +337,27 @@ int oracle_unpermute_combine(const uint16_t *y, int64_t n_perm, int64_t H, const
                 out_bf16[t * H + h] = f32_to_bf16(acc);
         }
     free(inv);
+    return 0;
+}
+
+/*
+ * SwiGLU of rows [a | b] (bf16 bit patterns), atorch/modules/moe/grouped_gemm_moe.py:331-334:
+ * torch.chunk(x, 2, -1); F.silu(x[0]) * x[1].  Two torch ops on bf16 tensors: silu is evaluated in
+ * fp32 as x / (1 + exp(-x)) and rounded to bf16, the product is formed in fp32 and rounded to bf16.
+ * The fp32 formula is followed operation by operation with a correctly rounded expf (so exp(-x)
+ * overflows to inf, and silu to -0, below about -88.7 as it does in fp32); an implementation whose
+ * expf is off by an ulp may differ by one bf16 unit in the last place on rare inputs.
+ */
+int oracle_swiglu_bf16(const uint16_t *fc1, int64_t rows, int64_t F, int64_t ld, uint16_t *h) {
+    if (rows < 0 || F < 0 || ld < 2 * F) return 1;
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < F; c++) {
+            const float a = bf16_to_f32(fc1[r * ld + c]);
+            const float b = bf16_to_f32(fc1[r * ld + F + c]);
+            const float e = (float)exp(-(double)a); /* correctly rounded expf; overflows to inf like fp32 */
+            const float sl32 = a / (1.0f + e);
+            const float sl = bf16_to_f32(f32_to_bf16(sl32));
+            h[r * F + c] = f32_to_bf16(sl * b);
+        }
     return 0;
 }

@@ -54,6 +54,7 @@ def lib() -> ctypes.CDLL:
         L.oracle_fp8_gemm.argtypes = [vp, i64, vp, i64, i64, vp, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci]
         L.oracle_permute_indices.argtypes = [vp, i64, i64, vp, vp]
         L.oracle_unpermute_combine.argtypes = [vp, i64, i64, vp, vp, ci, i64, i64, vp, vp]
+        L.oracle_swiglu_bf16.argtypes = [vp, i64, i64, i64, vp]
         for name in (
             "oracle_tile_quant",
             "oracle_block_quant",
@@ -165,6 +166,22 @@ def tile_quant_t_grouped(
         "tile_quant_t_grouped",
     )
     return q_t, s_t
+
+
+def swiglu(fc1: torch.Tensor) -> torch.Tensor:
+    """grouped_gemm_moe.py:331-334 on bf16 rows [a | b]: bf16(bf16(silu(a)) * b)."""
+    assert fc1.dtype == torch.bfloat16 and fc1.dim() == 2
+    x = fc1.contiguous().view(torch.int16)
+    rows, two_f = x.shape
+    h = torch.empty((rows, two_f // 2), dtype=torch.int16)
+    _chk(lib().oracle_swiglu_bf16(_p(x), rows, two_f // 2, two_f, _p(h)), "swiglu")
+    return h.view(torch.bfloat16)
+
+
+def torch_swiglu(fc1: torch.Tensor) -> torch.Tensor:
+    """The reference's own two torch ops (CPU)."""
+    a, b = torch.chunk(fc1, 2, dim=-1)
+    return torch.nn.functional.silu(a) * b
 
 
 def dequant(q: torch.Tensor, s: torch.Tensor) -> torch.Tensor:

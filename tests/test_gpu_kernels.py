@@ -23,6 +23,72 @@ def _u8(t):
 
 
 # ------------------------------------------------------------------------------------------
+# SwiGLU fused into the quantisation of the intermediate activations
+# ------------------------------------------------------------------------------------------
+def _ulp_diff(a, b):
+    return (a.view(torch.int16).int() - b.view(torch.int16).int()).abs()
+
+
+def test_swiglu_over_all_bf16_values(oracle, dev):
+    """h from the fused kernel against the oracle for every finite bf16 value of a: the kernel
+    evaluates silu in fp32 (x / (1 + expf(-x))), the oracle rounds the exact value, so single-ulp
+    differences of the bf16 result are allowed on a small fraction of inputs; nothing larger."""
+    from atorch_amd import kernels
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    a = bits[bits.float().abs() < 2.0**100]  # larger values overflow the product: out of the quantiser's contract
+    a = a[: a.numel() // 128 * 128].view(-1, 128)
+    g = torch.Generator().manual_seed(4)
+    b = (torch.randn(a.shape, generator=g) * 2).bfloat16()
+    fc1 = torch.cat([a, b], dim=1).contiguous()
+    q, s, h = kernels.swiglu_tile_quant(fc1.to(dev), return_activation=True)
+    ho = oracle.swiglu(fc1)
+    d = _ulp_diff(h.cpu(), ho)
+    # +-0 differ by 0x8000 as integers but are equal values
+    d = torch.where(h.cpu().float() == ho.float(), torch.zeros_like(d), d)
+    assert int(d.max()) <= 1, int(d.max())
+    assert float((d > 0).float().mean()) < 2e-3
+    # the codes and scales are exactly the quantisation of the kernel's own activation
+    qo, so = oracle.tile_quant(h.cpu())
+    assert torch.equal(_u8(q), qo) and torch.equal(s.cpu(), so)
+
+
+@pytest.mark.parametrize("M,F,E", [(300, 256, 3), (1000, 1408 // 128 * 128, 5)])
+def test_swiglu_quant_dual_grouped(oracle, dev, M, F, E):
+    """The fused kernel equals SwiGLU followed by the dual (row + transposed) grouped quantisation:
+    its outputs are bit-identical to tile_quant_dual_grouped applied to its own activation, which
+    is within one bf16 ulp of the oracle's."""
+    from atorch_amd import kernels
+
+    splits = ragged_splits(M, E, seed=5)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    fc1 = randn_bf16((M, 2 * F), 6, std=2.0)
+    q, s, q_t, s_t, h = kernels.swiglu_tile_quant_dual_grouped(fc1.to(dev), goff, E, return_activation=True)
+    ho = oracle.swiglu(fc1)
+    d = _ulp_diff(h.cpu(), ho)
+    d = torch.where(h.cpu().float() == ho.float(), torch.zeros_like(d), d)
+    assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 2e-3
+    q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(h, goff, E, ld_t=q_t.shape[1])
+    assert torch.equal(_u8(q), _u8(q2)) and torch.equal(s, s2)
+    # columns / scale rows past the padded total are not written by either kernel
+    ptot = kernels.padded_total(splits)
+    assert torch.equal(s_t[: ptot // TILE], s_t2[: ptot // TILE])
+    assert torch.equal(_u8(q_t[:, :ptot]), _u8(q_t2[:, :ptot]))
+    # transposed only
+    _, _, q_t3, s_t3 = kernels.swiglu_tile_quant_dual_grouped(fc1.to(dev), goff, E, ld_t=q_t.shape[1], rowwise=False)
+    assert torch.equal(_u8(q_t3[:, :ptot]), _u8(q_t[:, :ptot])) and torch.equal(s_t3[: ptot // TILE], s_t[: ptot // TILE])
+
+
+def test_swiglu_quant_rejects_bad_shapes(dev):
+    from atorch_amd import kernels
+
+    with pytest.raises(AssertionError):
+        kernels.swiglu_tile_quant(torch.zeros(4, 384, dtype=torch.bfloat16, device=dev))  # F = 192
+    with pytest.raises(AssertionError):
+        kernels.swiglu_tile_quant(torch.zeros(4, 256, dtype=torch.float32, device=dev))
+
+
+# ------------------------------------------------------------------------------------------
 # a1: 1x128 quant
 # ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

@@ -341,3 +341,26 @@ def test_grouped_linear_oracle_against_fp64_autograd(oracle):
         assert close(r["wgrad"][e], wd[e].grad)
     assert torch.all(r["wgrad"][1] == 0)
     assert math.isclose(float(r["bgrad"][0].sum()), float(dy[:128].float().sum()), rel_tol=1e-5)
+
+
+def test_swiglu_matches_torch_and_closed_forms(oracle):
+    """grouped_gemm_moe.py:331-334: F.silu(a) * b on bf16 tensors.  Over every finite bf16 value of a
+    (b = 1 and b random) the oracle equals torch's CPU ops; silu(0) = 0, silu(x) = x for large x and
+    -0 for very negative x; and h tracks a * sigmoid(a) * b computed in float64 within bf16 rounding."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    a = bits[torch.isfinite(bits.float())]
+    n = a.numel() // 128 * 128
+    a = a[:n].view(-1, 128)
+    g = torch.Generator().manual_seed(3)
+    for b in (torch.ones_like(a), (torch.randn(a.shape, generator=g) * 2).bfloat16()):
+        fc1 = torch.cat([a, b], dim=1).contiguous()
+        h = oracle.swiglu(fc1)
+        t = oracle.torch_swiglu(fc1)
+        assert torch.equal(h.view(torch.int16), t.view(torch.int16))
+        exact = a.double() * torch.sigmoid(a.double()) * b.double()
+        ok = (exact.abs() < 1e37) & (exact.abs() > 1e-30) & (a.double() > -87.0)  # below: exp(-a) overflows in fp32
+        rel = ((h.double() - exact).abs() / exact.abs())[ok]
+        assert float(rel.max()) < 2.0**-7  # two bf16 roundings
+    z = torch.tensor([[0.0, -0.0, 80.0, -120.0] + [0.0] * 124 + [3.0] * 128]).bfloat16()
+    h = oracle.swiglu(z)
+    assert h[0, 0].item() == 0.0 and h[0, 2].item() == 240.0 and h[0, 3].item() == 0.0
