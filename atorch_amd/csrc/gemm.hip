@@ -130,7 +130,7 @@ __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
 template <int MODE, bool R_PER_ROW, typename OUT, typename C>
 __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kernel(const GemmParams p) {
   constexpr int BM = C::BM, BN = C::BN, NT = C::NT;
-  // LDS: two stages, each [L tile | R tile] of 128-byte rows, then the two stages' scales
+  // LDS: two stages of an L tile and an R tile of 128-byte rows, then the two stages' scales
   // ([L rows | R rows or R blocks | unused], NT floats each).  After the contraction loop the same
   // memory stages the output tile for the row-contiguous stores of the epilogue.
   constexpr int kStage = (BM + BN) * kBK;
@@ -141,10 +141,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   static_assert(NT == 2 * BM, "two threads fetch the 32 bytes of a row's scale batch");
   __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4 + 2 * kLsBatch];
   __shared__ int slot;
+  // both L stages first, then both R stages: every fragment of a side is within 64 KB of one base
+  // address, so the stage and the sub-tile row go into the immediate offset of the LDS reads
   uint8_t* const Lbuf0 = lds;
-  uint8_t* const Rbuf0 = lds + BM * kBK;
-  uint8_t* const Lbuf1 = lds + kStage;
-  uint8_t* const Rbuf1 = lds + kStage + BM * kBK;
+  uint8_t* const Lbuf1 = lds + BM * kBK;
+  uint8_t* const Rbuf0 = lds + 2 * BM * kBK;
+  uint8_t* const Rbuf1 = lds + 2 * BM * kBK + BN * kBK;
+  static_assert(2 * BM * kBK <= 65536 && 2 * BN * kBK <= 65536, "immediate LDS offsets are 16 bits");
   float* const Sc0 = reinterpret_cast<float*>(lds + 2 * kStage);
   float* const Sc1 = Sc0 + NT;
   float* const LsB0 = Sc1 + NT;  // scale batches (kRaggedRows)
@@ -152,9 +155,11 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   const int tid = threadIdx.x;
 #ifdef AAMD_GEMM_TIMING
   // measurement build: six time stamps per workgroup go where the bias would be read from
-  unsigned long long stamp[6];
+  // (plus the constant-rate clock at both ends of the workgroup and the hardware ids of the compute unit)
+  unsigned long long stamp[8];
   stamp[0] = __builtin_readcyclecounter();
-#define AAMD_STAMP(i) stamp[i] = __builtin_readcyclecounter()
+  stamp[6] = __builtin_amdgcn_s_memrealtime();
+#define AAMD_STAMP(i) stamp[i] = __builtin_readcyclecounter(); if (i == 4) stamp[7] = (unsigned long long)__builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11)) | ((unsigned long long)__builtin_amdgcn_s_getreg((20) | (0 << 6) | (31 << 11)) << 32)
 #else
 #define AAMD_STAMP(i)
 #endif
@@ -370,6 +375,18 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     for (int c = 0; c < 2; c++) chk[h][c] = ((4 * h + 2 * hg + c) ^ sw) << 4;
   const int wrow0 = wr * C::WTR * 32;            // first R row of this wave inside the tile
   const int wlrow0 = wl * C::WTL * 32;           // first L row of this wave inside the tile
+  // LDS byte addresses of this lane's four chunks in its row of the wave's first sub-tile, stage 0.
+  // Kept opaque: every fragment read is one of these plus a compile-time offset.
+  uint32_t la[2][2], ra[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      la[h][c] = (uint32_t)(uintptr_t)(lds_ptr_t)Lbuf0 + (uint32_t)((wlrow0 + l32) * kBK + chk[h][c]);
+      ra[h][c] = (uint32_t)(uintptr_t)(lds_ptr_t)Rbuf0 + (uint32_t)((wrow0 + l32) * kBK + chk[h][c]);
+      asm volatile("" : "+v"(la[h][c]));
+      asm volatile("" : "+v"(ra[h][c]));
+    }
   const bool wave_active = wrow0 < rvalid;        // whole wave in or out: rvalid % 128 == 0
 
   v16f acc[C::WTR][C::WTL];
@@ -387,38 +404,51 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // the workgroup barrier.  Branch free: waves outside a partial R tile compute on clamped
   // rows and skip only the final store.
   constexpr int NTILES = C::WTR * C::WTL;
-  auto compute = [&](int kb, const uint8_t* Lt, const uint8_t* Rt, const float* Sct, auto&& after_l_reads,
-                     auto&& per_tile) {
+  auto compute = [&](int kb, int stage, const float* Sct, auto&& after_l_reads, auto&& per_tile) {
     __builtin_amdgcn_sched_barrier(0);
     // L scale of tile row r: Lsc[r * lsc_stride]
     const int bsel = kb >> 3;
     const float* Lsc = batch ? LsB0 + (bsel & 1) * (BM * 8) + (kb - batch_start(bsel)) : Sct;
     const int lsc_stride = batch ? 8 : 1;
     const float* Rsc = Sct + BM;
-    auto load_frag = [&](const uint8_t* T, int row, int h) {
+    // fragment of sub-tile row `sub` (32 rows each) of one side, K half h
+    typedef const __attribute__((address_space(3))) v4i* lds_v4i_t;
+    auto load_frag = [&](const uint32_t (&base)[2][2], int rows_per_stage, int sub, int h) {
 #if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE >= 5
       { v8i f; asm volatile("" : "=v"(f)); return f; }  // measurement build: operands from nowhere
 #endif
-      const v4i lo = *reinterpret_cast<const v4i*>(T + row * kBK + chk[h][0]);
-      const v4i hi = *reinterpret_cast<const v4i*>(T + row * kBK + chk[h][1]);
+      const uint32_t delta = (uint32_t)((stage * rows_per_stage + sub * 32) * kBK);
+      const v4i lo = *(lds_v4i_t)(uintptr_t)(base[h][0] + delta);
+      const v4i hi = *(lds_v4i_t)(uintptr_t)(base[h][1] + delta);
       return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
     v8i lf[C::WTL][2];
     float cs[C::WTL];
     const float rblk = R_PER_ROW ? 1.f : Rsc[wrow0 / kTile];
+    v8i rf[2][2];
+    // LDS reads in the order of first use: the first MFMA waits for two fragments only, the rest
+    // arrive in its shadow
+    lf[0][0] = load_frag(la, BM, 0, 0);
+    rf[0][0] = load_frag(ra, BN, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    lf[0][1] = load_frag(la, BM, 0, 1);
+    rf[0][1] = load_frag(ra, BN, 0, 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < C::WTL; j++) {
       const int row = wlrow0 + j * 32 + l32;
-      lf[j][0] = load_frag(Lt, row, 0);
-      lf[j][1] = load_frag(Lt, row, 1);
+      if (j > 0) {
+        lf[j][0] = load_frag(la, BM, j, 0);
+        lf[j][1] = load_frag(la, BM, j, 1);
+      }
       cs[j] = Lsc[row * lsc_stride] * rblk;
     }
-    v8i rf[2][2];
     v4f rs[2][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
     auto load_r = [&](int i) {
-      const int row = wrow0 + i * 32 + l32;
-      rf[i & 1][0] = load_frag(Rt, row, 0);
-      rf[i & 1][1] = load_frag(Rt, row, 1);
+      if (i > 0) {
+        rf[i & 1][0] = load_frag(ra, BN, i, 0);
+        rf[i & 1][1] = load_frag(ra, BN, i, 1);
+      }
       if constexpr (R_PER_ROW) {
 #pragma unroll
         for (int q = 0; q < 4; q++)
@@ -503,13 +533,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     int kb = 0;
     for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
       if (kLoads) dma(kb + 1, Lbuf1, Rbuf1, Sc1);
-      if (kMath) compute(kb, Lbuf0, Rbuf0, Sc0, nothing, no_feed);
+      if (kMath) compute(kb, 0, Sc0, nothing, no_feed);
       dma_wait_and_sync();
       if (kLoads) dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
-      if (kMath) compute(kb + 1, Lbuf1, Rbuf1, Sc1, nothing, no_feed);
+      if (kMath) compute(kb + 1, 1, Sc1, nothing, no_feed);
       dma_wait_and_sync();
     }
-    if (kb < nkb) compute(kb, Lbuf0, Rbuf0, Sc0, nothing, no_feed);  // odd number of steps
+    if (kb < nkb) compute(kb, 0, Sc0, nothing, no_feed);  // odd number of steps
   } else {
     // The L fragments of a step sit in registers for the whole step, so the L half of a stage is
     // free as soon as every wave has read it: an extra barrier after those reads lets the L tile of
@@ -528,23 +558,23 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       AAMD_STAMP(2);
       wait_all_but_newest_l();
       AAMD_STAMP(3);
-      auto step = [&](int kb, uint8_t* Lc, uint8_t* Rc, float* Sc, uint8_t* Rn, float* Sn) {
+      auto step = [&](int kb, int stage, uint8_t* Lc, float* Sc, uint8_t* Rn, float* Sn) {
         if (kLoads) dmaR(kclamp(kb + 1), Rn, Sn);
         auto mid = [&]() {
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
           if (kLoads) dmaL(kclamp(kb + 2), Lc, Sc);
         };
-        if (kMath) compute(kb, Lc, Rc, Sc, mid, no_feed);
+        if (kMath) compute(kb, stage, Sc, mid, no_feed);
         else mid();
         if (kLoads) wait_all_but_newest_l();
         else asm volatile("s_barrier" ::: "memory");
       };
       int kb = 0;
       for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
-        step(kb, Lbuf0, Rbuf0, Sc0, Rbuf1, Sc1);
-        step(kb + 1, Lbuf1, Rbuf1, Sc1, Rbuf0, Sc0);
+        step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
+        step(kb + 1, 1, Lbuf1, Sc1, Rbuf0, Sc0);
       }
-      if (kb < nkb) step(kb, Lbuf0, Rbuf0, Sc0, Rbuf1, Sc1);
+      if (kb < nkb) step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
     }
   }
@@ -642,9 +672,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   stamp[1] = __builtin_readcyclecounter();  // epilogue issued (overwrites the group-lookup stamp)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   stamp[5] = __builtin_readcyclecounter();
+  stamp[2] = __builtin_amdgcn_s_memrealtime();  // constant-rate clock at the end (overwrites the loads-issued stamp)
   if (tid == 0 && p.bias != nullptr) {
-    unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 6;
-    for (int i = 0; i < 6; i++) dst[i] = stamp[i];
+    unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 8;
+    for (int i = 0; i < 8; i++) dst[i] = stamp[i];
   }
 #endif
 }
