@@ -120,6 +120,17 @@ typedef Cfg<2, 2, 2, 2, 3> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two wor
 typedef Cfg<2, 4, 4, 2, AAMD_LARGE_PRB, AAMD_LARGE_LAHEAD> CfgLarge;  // 512 threads, 256 (L) x 256 (R); one product buffer: 256 registers per lane
 typedef Cfg<2, 4, 2, 2> CfgWgrad;  // 512 threads, 256 (L) x 128 (R): room for the per-row R scales
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
+// expression inside the body.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 // A 64-bit offset the compiler can keep in scalar registers (it is the same in every lane).
 __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)(uint64_t)v);
@@ -321,24 +332,34 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   };
   // One wave instruction of the L (R) tile of a step; the last one of a half also carries that
   // half's scale loads.  L half: the L tile and, from the waves that own them, the L scales.
-  auto dmaL_one = [&](int n, int kb, uint8_t* Ld, float* Sd) {
+  auto dmaL_tile = [&](int n, int kb, uint8_t* Ld) {
     const uint8_t* lb = Lbase + (int64_t)kb * kBK;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  ::"v"(ltail[n] ? voffLt : voffL), "s"(lb + lslab[n]),
                    "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
                  : "memory");
-    if (n == C::LCH - 1 && l_side && step_scale) dma_scale(kb, Sd);
   };
-  auto dmaR_one = [&](int n, int kb, uint8_t* Rd, float* Sd) {
+  auto dmaL_scales = [&](int kb, float* Sd) {
+    if (l_side && step_scale) dma_scale(kb, Sd);
+  };
+  auto dmaR_tile = [&](int n, int kb, uint8_t* Rd) {
     const uint8_t* rb = Rbase + (int64_t)kb * kBK;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  ::"v"(voffR), "s"(rb + rslab[n]),
                    "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
                  : "memory");
-    if (n == C::RCH - 1) {
-      if (!l_side) dma_scale(kb, Sd);
-      if (batch && (kb & 7) == 0) dma_scale_batch(kb >> 3);  // lands a step before its first use
-    }
+  };
+  auto dmaR_scales = [&](int kb, float* Sd) {
+    if (!l_side) dma_scale(kb, Sd);
+    if (batch && (kb & 7) == 0) dma_scale_batch(kb >> 3);  // lands a step before its first use
+  };
+  auto dmaL_one = [&](int n, int kb, uint8_t* Ld, float* Sd) {
+    dmaL_tile(n, kb, Ld);
+    if (n == C::LCH - 1) dmaL_scales(kb, Sd);
+  };
+  auto dmaR_one = [&](int n, int kb, uint8_t* Rd, float* Sd) {
+    dmaR_tile(n, kb, Rd);
+    if (n == C::RCH - 1) dmaR_scales(kb, Sd);
   };
   auto dmaL = [&](int kb, uint8_t* Ld, float* Sd) {
 #pragma unroll
@@ -476,9 +497,9 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     // Issue order per sub-tile, kept by full scheduling barriers: first MFMA, half of the previous
     // sub-tile's fold, second MFMA, the other half, then the LDS reads of the next R row.  Each MFMA
     // (16 passes) covers its own issue plus eight FMAs of another sub-tile.
-#pragma unroll
-    for (int t = 0; t < NTILES; t++) {
-      const int i = t / C::WTL, j = t % C::WTL;
+    static_for<NTILES>([&](auto T) {
+      constexpr int t = decltype(T)::value;
+      constexpr int i = t / C::WTL, j = t % C::WTL;
       __builtin_amdgcn_sched_barrier(0);
       pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
       __builtin_amdgcn_sched_barrier(0);
@@ -497,9 +518,9 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       __builtin_amdgcn_sched_barrier(0);
       // every L fragment has been an MFMA operand by now, so it has left the LDS: the hook (a
       // barrier and the next L loads) costs no extra wait here
+      per_tile(T);
       if (t == C::WTL - 1) after_l_reads();
-      per_tile(t);
-    }
+    });
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = NTILES - D; t < NTILES; t++) {
@@ -524,9 +545,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #endif
   constexpr bool kLoads = AAMD_GEMM_ABLATE != 1 && AAMD_GEMM_ABLATE < 4, kMath = AAMD_GEMM_ABLATE < 2 || AAMD_GEMM_ABLATE >= 4;
   auto nothing = [] {};
-  auto no_feed = [](int) {};
-  // (Spreading the loads of a step over its sub-tiles instead of issuing them in one burst after
-  // the barrier measured slower: they then have less time to arrive.)
+  auto no_feed = [](auto) {};
+  // Two workgroups per CU: the loads of a step go out in one burst after the barrier (issued a few
+  // at a time behind the sub-tiles they measured 6 % slower here: they have less time to arrive,
+  // and the other workgroup already fills the issue gap).
   if constexpr (!C::LAHEAD) {
     if (nkb > 0) dma(0, Lbuf0, Rbuf0, Sc0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -559,12 +581,31 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       wait_all_but_newest_l();
       AAMD_STAMP(3);
       auto step = [&](int kb, int stage, uint8_t* Lc, float* Sc, uint8_t* Rn, float* Sn) {
-        if (kLoads) dmaR(kclamp(kb + 1), Rn, Sn);
+        // One workgroup per CU: a burst of loads right after the barrier holds up every wave's first
+        // MFMAs, so the tile loads go out a few at a time behind the first sub-tiles (measured 4-5 %
+        // faster): the R tile before the barrier that frees the L half, the L tile after it.  The
+        // scale loads sit behind uniform branches and stay at the head of their group: control flow
+        // inside the sub-tile sequence costs the register allocator dearly.
+        constexpr int RT = C::WTL, RPER = C::RCH / RT;
+        static_assert(C::RCH % RT == 0 && RT + C::LCH <= NTILES, "spread schedule");
+        const int kr = kclamp(kb + 1), kl = kclamp(kb + 2);
         auto mid = [&]() {
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
-          if (kLoads) dmaL(kclamp(kb + 2), Lc, Sc);
+          if (kLoads && !kMath) dmaL(kl, Lc, Sc);
+          else if (kLoads) dmaL_scales(kl, Sc);
         };
-        if (kMath) compute(kb, stage, Sc, mid, no_feed);
+        auto feed = [&](auto T) {
+          constexpr int t = decltype(T)::value;
+          if (!kLoads) return;
+          if constexpr (t < RT) {
+            static_for<RPER>([&](auto N) { dmaR_tile(t * RPER + decltype(N)::value, kr, Rn); });
+          } else if constexpr (t < RT + C::LCH) {
+            dmaL_tile(t - RT, kl, Lc);
+          }
+        };
+        if (kLoads && !kMath) dmaR(kr, Rn, Sn);
+        else if (kLoads) dmaR_scales(kr, Sn);
+        if (kMath) compute(kb, stage, Sc, mid, feed);
         else mid();
         if (kLoads) wait_all_but_newest_l();
         else asm volatile("s_barrier" ::: "memory");
