@@ -88,13 +88,11 @@ __device__ __forceinline__ float scale_from_amax(float amax, float eps) {
 }
 
 // Two floats -> two e4m3fn codes in the low or high half of `old` (RNE, v_cvt_pk_fp8_f32).
-// Inputs are clamped to +-448 first: by construction |x/s| <= 448(1+2^-23), which RNE maps to
-// 448 anyway, so the clamp never changes an in-contract result but keeps the encoder away
-// from its overflow behaviour.
+// No clamp ahead of the encoder: a quotient x / s with s = RN(max(amax, eps) / 448) and
+// |x| <= amax is at most 448 (1 + 2^-23), which RNE maps to 448 (the encoder's own overflow
+// handling starts above 464).
 template <bool HI>
 __device__ __forceinline__ int pack2_fp8(float a, float b, int old) {
-  a = __builtin_amdgcn_fmed3f(a, -kFp8Max, kFp8Max);
-  b = __builtin_amdgcn_fmed3f(b, -kFp8Max, kFp8Max);
   return __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, HI);
 }
 
@@ -105,7 +103,7 @@ __device__ __forceinline__ int pack2_fp8(float a, float b, int old) {
 // range scaling).  Scales whose reciprocal could leave the normal range take the plain division.
 // The scheme is used where it has been checked against the plain division over its whole domain:
 // bf16 values divided by the scale of a bf16 maximum (amax / 448).  fp32 inputs and scales that
-// come from an eps clamp take the plain division.  The sign of a zero quotient is taken from x.
+// come from an eps clamp take the plain division.
 struct Divider {
   float s, y;
   bool plain;
@@ -119,28 +117,36 @@ __device__ __forceinline__ Divider make_divider(float s, bool force_plain) {
   d.plain = force_plain || !(s > 0x1p-100f && s < 0x1p100f);
   return d;
 }
-__device__ __forceinline__ float div_by(float x, const Divider& d) {
+__device__ __forceinline__ float neg_div_by(float x, const Divider& d) {
   const float q = x * d.y;
   const float r = __builtin_fmaf(-d.s, q, x);
-  return __builtin_copysignf(__builtin_fmaf(r, d.y, q), x);  // s > 0
+  // -(q + r*y) as (r)(-y) + (-q): the same rounding, and a zero keeps the (flipped) sign of x: r is
+  // +0 then, so the sum is (-0) + (-q).  The caller flips the sign bits of the packed codes.
+  return __builtin_fmaf(r, -d.y, -q);
 }
 
 // 8 values / one scale -> 8 codes in two dwords, quotients rounded as by IEEE division.
 __device__ __forceinline__ v2i quant8(const float* v, float s, bool force_plain) {
   const Divider d = make_divider(s, force_plain);
   float t[8];
+  auto pack = [&]() {
+    v2i o;
+    int w = pack2_fp8<false>(t[0], t[1], 0);
+    o[0] = pack2_fp8<true>(t[2], t[3], w);
+    w = pack2_fp8<false>(t[4], t[5], 0);
+    o[1] = pack2_fp8<true>(t[6], t[7], w);
+    return o;
+  };
   if (__builtin_expect(d.plain, 0)) {
 #pragma unroll
     for (int i = 0; i < 8; i++) t[i] = v[i] / s;
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; i++) t[i] = div_by(v[i], d);
+    return pack();
   }
-  v2i o;
-  int w = pack2_fp8<false>(t[0], t[1], 0);
-  o[0] = pack2_fp8<true>(t[2], t[3], w);
-  w = pack2_fp8<false>(t[4], t[5], 0);
-  o[1] = pack2_fp8<true>(t[6], t[7], w);
+#pragma unroll
+  for (int i = 0; i < 8; i++) t[i] = neg_div_by(v[i], d);
+  v2i o = pack();
+  o[0] ^= (int)0x80808080u;  // the quotients were negated: flip the sign bit of every code
+  o[1] ^= (int)0x80808080u;
   return o;
 }
 
