@@ -157,6 +157,18 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
   for (int i = 0; i < 8; i++) raw[i].get(v[i]);
 }
 
+// the staged 128 x 128 code tile written as rows of 128 bytes, one 16-byte store per lane
+__device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t* __restrict__ out, int64_t ld_out) {
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < 4; n++) {
+    const int idx = threadIdx.x + 256 * n;
+    const int r = idx >> 3, ch = idx & 7;
+    __builtin_nontemporal_store(*reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16),
+                                reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16));
+  }
+}
+
 // codes of the 8x8 register block, transposed through LDS, written as rows of 128 bytes:
 // out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
 __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const float* cs, uint8_t* tile_t,
@@ -169,14 +181,7 @@ __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const f
     for (int i = 0; i < 8; i++) col[i] = v[i][j];
     *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cs[j], plain_div);
   }
-  __syncthreads();
-#pragma unroll
-  for (int n = 0; n < 4; n++) {
-    const int idx = threadIdx.x + 256 * n;
-    const int r = idx >> 3, ch = idx & 7;
-    __builtin_nontemporal_store(*reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16),
-                                reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16));
-  }
+  store_staged_tile(tile_t, out, ld_out);
 }
 
 template <typename IN>
@@ -186,9 +191,11 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
     u16* __restrict__ h_out) {
   const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
-  __shared__ float part[16][kTile];
-  __shared__ float cscale[kTile];
+  // the per-row-group column maxima are dead before the transposed codes are staged: one region
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
+  static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_t), "the column maxima fit in the staging region");
+  float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
+  __shared__ float cscale[kTile];
   __shared__ int slot;
 
   const int kc = blockIdx.x, pt = blockIdx.y;
@@ -242,6 +249,26 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   store_transposed(v, cs, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t, plain_div);
 }
 
+// The 8x8 byte matrix held as eight rows of two dwords, transposed with byte permutes: cols[j]
+// holds byte j of rows 0..7.  (v_perm_b32 selects bytes 0-3 from its second source, 4-7 from the first.)
+__device__ __forceinline__ void transpose8x8_bytes(const v2i (&rows)[8], v2i (&cols)[8]) {
+#pragma unroll
+  for (int jb = 0; jb < 2; jb++)
+#pragma unroll
+    for (int ib = 0; ib < 2; ib++) {
+      const uint32_t a = (uint32_t)rows[4 * ib][jb], b = (uint32_t)rows[4 * ib + 1][jb];
+      const uint32_t c = (uint32_t)rows[4 * ib + 2][jb], d = (uint32_t)rows[4 * ib + 3][jb];
+      const uint32_t x0 = __builtin_amdgcn_perm(b, a, 0x05010400u);  // a0 b0 a1 b1
+      const uint32_t x1 = __builtin_amdgcn_perm(b, a, 0x07030602u);  // a2 b2 a3 b3
+      const uint32_t y0 = __builtin_amdgcn_perm(d, c, 0x05010400u);
+      const uint32_t y1 = __builtin_amdgcn_perm(d, c, 0x07030602u);
+      cols[4 * jb + 0][ib] = (int)__builtin_amdgcn_perm(y0, x0, 0x05040100u);  // a0 b0 c0 d0
+      cols[4 * jb + 1][ib] = (int)__builtin_amdgcn_perm(y0, x0, 0x07060302u);
+      cols[4 * jb + 2][ib] = (int)__builtin_amdgcn_perm(y1, x1, 0x05040100u);
+      cols[4 * jb + 3][ib] = (int)__builtin_amdgcn_perm(y1, x1, 0x07060302u);
+    }
+}
+
 template <typename IN>
 __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::elem* __restrict__ w,
                                                             int64_t expert_stride, int64_t N, int64_t K,
@@ -271,14 +298,20 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
     if (s_t != nullptr) s_t[((int64_t)e * nkb + kb) * nnb + nb] = sc;
   }
   uint8_t* qe = q + (int64_t)e * N * K + (int64_t)nb * kTile * K + (int64_t)kb * kTile;
+  v2i codes[8];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
-    __builtin_nontemporal_store(quant8(v[i], sc, plain_div), reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8));
+  for (int i = 0; i < 8; i++) {
+    codes[i] = quant8(v[i], sc, plain_div);
+    __builtin_nontemporal_store(codes[i], reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8));
+  }
   if (q_t != nullptr) {
-    float cs[8];
+    // one scale for the whole block: the transposed copy holds the same codes, so the 8x8 block of
+    // this thread is transposed bytewise instead of being quantised a second time
+    v2i cols[8];
+    transpose8x8_bytes(codes, cols);
 #pragma unroll
-    for (int j = 0; j < 8; j++) cs[j] = sc;
-    store_transposed(v, cs, tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, N, plain_div);
+    for (int j = 0; j < 8; j++) *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = cols[j];
+    store_staged_tile(tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, N);
   }
 }
 
