@@ -35,6 +35,10 @@ SIGNATURES = {
         _int,
         [_vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
     ),
+    "aamd_swiglu_bwd_quant_1x128_dual_grouped": (
+        _int,
+        [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+    ),
     "aamd_quant_128x128": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp]),
     "aamd_dequant": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _int, _vp]),
     "aamd_grouped_gemm_fp8_nt": (

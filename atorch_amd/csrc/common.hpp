@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "../../include/atorch_amd_fp8.h"
 
@@ -53,6 +54,12 @@ struct BF16 {
 // bf16 rows [a | b] of a gated linear unit: the element read at column c is
 // h = bf16(bf16(silu(a[c])) * b[c]) with b = a + gate_off (grouped_gemm_moe.py:331-334).
 struct GLU {
+  typedef u16 elem;
+};
+// Backward of the same unit: rows [a | b] plus the gradient dh of h; the element read at column c
+// of the [da | db] row is da = bf16(bf16(dh*b) * sig(a) * (1 + a*(1 - sig(a)))) or
+// db = bf16(dh * bf16(silu(a))), what autograd makes of the two torch ops on bf16 tensors.
+struct GLUB {
   typedef u16 elem;
 };
 struct F32 {

@@ -200,7 +200,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     const int in_grp = (int)(pid % width);
     lt = first + in_grp % gsz;
     rt = in_grp / gsz;
-#if defined(AAMD_GEMM_ABLATE) && (AAMD_GEMM_ABLATE == 3 || AAMD_GEMM_HOT)
+#if defined(AAMD_GEMM_ABLATE) && (AAMD_GEMM_ABLATE == 3 || AAMD_GEMM_HOT == 1)
     lt = 0; rt = 0;  // measurement build: every workgroup streams the same tile
 #endif
   }
@@ -242,6 +242,11 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // uniform tile bases + per-thread 32-bit offsets
   const uint8_t* Lbase = p.L + uniform_i64(l0 * p.ldl + (int64_t)kb0 * kBK);
   const uint8_t* Rbase = p.R + uniform_i64((int64_t)g * p.r_group_stride + r0 * p.ldr + (int64_t)kb0 * kBK);
+#if defined(AAMD_GEMM_HOT) && AAMD_GEMM_HOT == 2
+  Lbase = p.L;  // measurement build: every workgroup streams the same L tile
+#elif defined(AAMD_GEMM_HOT) && AAMD_GEMM_HOT == 3
+  Rbase = p.R;  // measurement build: every workgroup streams the same R tile
+#endif
   const float* Lsg = p.Ls + (int64_t)kb0 * p.ls_blk_stride;
   const float* Rsg = p.Rs + (int64_t)g * p.rs_group_stride + (int64_t)kb0 * p.rs_blk_stride;
 

@@ -4,7 +4,7 @@
 //
 // All of them stream HBM with 128-bit accesses; amax reductions over a 128-element tile run
 // inside one 16-lane DPP row.  Scales and codes are part of a bit-exact contract, so every
-// division is the IEEE one (no reciprocal tricks).
+// quotient is the correctly rounded one (the IEEE division or its checked three-instruction form).
 #include "common.hpp"
 
 namespace aamd {
@@ -61,6 +61,44 @@ struct Raw8<GLU> {
       const uint32_t h = pack_bf16x2(__uint_as_float(sl << 16) * fb[i], __uint_as_float(sl & 0xffff0000u) * fb[i + 1]);
       v[i] = __uint_as_float(h << 16);
       v[i + 1] = __uint_as_float(h & 0xffff0000u);
+    }
+  }
+};
+
+// SwiGLU backward on load.  The loader reads a, b (unless only db is wanted) and dh; get() yields
+// eight elements of da or of db.
+struct GluBwd8 {
+  v4i a, b, d;
+  __device__ __forceinline__ void load(const u16* pa, int64_t gate_off, const u16* pd, bool want_db) {
+    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pa));
+    d = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pd));
+    if (!want_db) b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pa + gate_off));
+    else b = v4i{0, 0, 0, 0};
+  }
+  __device__ __forceinline__ void zero() { a = b = d = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v, bool want_db) const {
+    float fa[8], fb[8], fd[8];
+    unpack8(a, fa);
+    unpack8(b, fb);
+    unpack8(d, fd);
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      float r0, r1;
+      // hardware exp2 and reciprocal, as in the forward loader
+      const float e0 = __expf(-fa[i]), e1 = __expf(-fa[i + 1]);
+      if (want_db) {
+        const uint32_t sl = pack_bf16x2(__fdividef(fa[i], 1.0f + e0), __fdividef(fa[i + 1], 1.0f + e1));
+        r0 = fd[i] * __uint_as_float(sl << 16);
+        r1 = fd[i + 1] * __uint_as_float(sl & 0xffff0000u);
+      } else {
+        const float sg0 = __fdividef(1.0f, 1.0f + e0), sg1 = __fdividef(1.0f, 1.0f + e1);
+        const uint32_t g = pack_bf16x2(fd[i] * fb[i], fd[i + 1] * fb[i + 1]);
+        r0 = (__uint_as_float(g << 16) * sg0) * (1.0f + fa[i] * (1.0f - sg0));
+        r1 = (__uint_as_float(g & 0xffff0000u) * sg1) * (1.0f + fa[i + 1] * (1.0f - sg1));
+      }
+      const uint32_t o = pack_bf16x2(r0, r1);
+      v[i] = __uint_as_float(o << 16);
+      v[i + 1] = __uint_as_float(o & 0xffff0000u);
     }
   }
 };
@@ -157,6 +195,24 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
   for (int i = 0; i < 8; i++) raw[i].get(v[i]);
 }
 
+// the same register tile of da (want_db false) or db for feature columns [f0, f0 + 128)
+__device__ __forceinline__ void load_tile_glu_bwd(const u16* __restrict__ fc1, int64_t ld, int64_t gate_off,
+                                                  const u16* __restrict__ dh, int64_t ld_dh, bool want_db,
+                                                  int rows_valid, float (&v)[8][8]) {
+  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+  GluBwd8 raw[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int r = gr * 8 + i;
+    if (r < rows_valid)
+      raw[i].load(fc1 + (int64_t)r * ld + c * 8, gate_off, dh + (int64_t)r * ld_dh + c * 8, want_db);
+    else
+      raw[i].zero();
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) raw[i].get(v[i], want_db);
+}
+
 // the staged 128 x 128 code tile written as rows of 128 bytes, one 16-byte store per lane
 __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t* __restrict__ out, int64_t ld_out) {
   __syncthreads();
@@ -189,7 +245,7 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
-    u16* __restrict__ h_out) {
+    u16* __restrict__ h_out, const u16* __restrict__ dh = nullptr, int64_t ld_dh = 0) {
   const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
@@ -198,7 +254,13 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   __shared__ float cscale[kTile];
   __shared__ int slot;
 
-  const int kc = blockIdx.x, pt = blockIdx.y;
+  int kc = blockIdx.x;
+  const int pt = blockIdx.y;
+  if constexpr (std::is_same<IN, GLUB>::value) {
+    // consecutive workgroups take the da and the db tile of the same features: the second one finds
+    // a and dh in the L2
+    kc = (blockIdx.x & 1) * (nt / 2) + (blockIdx.x >> 1);
+  }
   const int g = find_group(tile_off, E, pt, &slot);
   if (g >= E) return;
   const int64_t cols = (int64_t)nt * kTile;
@@ -208,7 +270,14 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
 
   float v[8][8];
-  load_tile<IN>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
+  if constexpr (std::is_same<IN, GLUB>::value) {
+    const int half = nt / 2;  // output column tiles [0, half) are da, [half, nt) are db
+    const bool want_db = kc >= half;
+    const int64_t f0 = (int64_t)(want_db ? kc - half : kc) * kTile;
+    load_tile_glu_bwd(x + m0 * ldx + f0, ldx, gate_off, dh + m0 * ld_dh + f0, ld_dh, want_db, mvalid, v);
+  } else {
+    load_tile<IN>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
+  }
 
   // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
   float cm[8];
@@ -518,6 +587,36 @@ extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, 
   quant_dual_grouped_kernel<GLU><<<grid, block, 0, st>>>((const u16*)fc1, ld, (int)(F / kTile), group_offsets, tile_ws, E,
                                                          q, s, q_t, s_t, ld_t, 0.f, F, (u16*)h_out);
   AAMD_LAUNCH_CHECK("swiglu_quant_dual_grouped");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t ld_dh, const void* fc1, int64_t ld,
+                                                        int64_t M, int64_t F, const int64_t* group_offsets, int E,
+                                                        int32_t* tile_ws, void* g_out, uint8_t* q, float* s,
+                                                        uint8_t* q_t, float* s_t, int64_t ld_t, void* stream) {
+  AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "swiglu_bwd_quant_dual: F=%lld must be a multiple of 128", (long long)F);
+  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld_dh >= F && ld_dh % 8 == 0, "swiglu_bwd_quant_dual: bad ld=%lld / ld_dh=%lld",
+               (long long)ld, (long long)ld_dh);
+  AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "swiglu_bwd_quant_dual: group_offsets / tile_ws required");
+  AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "swiglu_bwd_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
+  AAMD_REQUIRE((q == nullptr) == (s == nullptr), "swiglu_bwd_quant_dual: q and s go together");
+  AAMD_REQUIRE(q_t && s_t, "swiglu_bwd_quant_dual: q_t / s_t required");
+  if (F == 0) return AAMD_OK;
+  const int64_t max_tiles = M / kTile + E;
+  const int64_t grid_tiles = ld_t / kTile < max_tiles ? ld_t / kTile : max_tiles;
+  if (grid_tiles == 0) return AAMD_OK;
+  AAMD_REQUIRE(dh && fc1, "swiglu_bwd_quant_dual: null input");
+  AAMD_REQUIRE(aligned16(fc1) && aligned16(dh) && aligned16(q_t) && (!q || aligned16(q)) && aligned16(g_out),
+               "swiglu_bwd_quant_dual: pointers must be 16-byte aligned");
+  AAMD_REQUIRE(grid_tiles <= 65535, "swiglu_bwd_quant_dual: more than 65535 token tiles");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
+  if (rc) return rc;
+  const int nt = (int)(2 * F / kTile);
+  dim3 grid((unsigned)nt, (unsigned)grid_tiles), block(256);
+  quant_dual_grouped_kernel<GLUB><<<grid, block, 0, st>>>((const u16*)fc1, ld, nt, group_offsets, tile_ws, E, q, s, q_t, s_t,
+                                                          ld_t, 0.f, F, (u16*)g_out, (const u16*)dh, ld_dh);
+  AAMD_LAUNCH_CHECK("swiglu_bwd_quant_dual_grouped");
   return AAMD_OK;
 }
 

@@ -12,8 +12,9 @@ with weights ``w1 [E, 2F, H]`` (``transpose_w1=True``, the default) or ``[E, H, 
 forward: the first GEMM's output is read once by a kernel that applies SwiGLU and writes the fp8
 codes and scales the second GEMM (and, under autograd, its weight-gradient GEMM) consume.
 
-Backward recomputes SwiGLU's pieces from the saved first-GEMM output with torch ops (bf16, the
-reference's own arithmetic) and runs the four gradient GEMMs on the fp8 kernels.
+Backward: the gradient through SwiGLU is computed from the saved first-GEMM output by the kernel
+that quantises it (same fusion, autograd's bf16 arithmetic), and the four gradient GEMMs run on
+the fp8 kernels.
 """
 import torch
 
@@ -61,14 +62,8 @@ class _Fp8SwigluMlp(torch.autograd.Function):
         # through the second linear: dh = dy @ w2^T ([M, F]); dw2[f, h] = sum_m h[m, f] dy[m, h]
         dh = kernels.grouped_gemm_nt(qdy, sdy, q2, s2, goff, out_dtype=torch.bfloat16)
         dw2 = kernels.grouped_gemm_wgrad(qh_t, sh_t, qdy_t, sdy_t, goff, out_dtype=w2_dtype)
-        # through SwiGLU, with the reference's torch arithmetic on bf16 tensors
-        a, b = torch.chunk(fc1, 2, dim=-1)
-        sig = torch.sigmoid(a.float())
-        sl = torch.nn.functional.silu(a)
-        db = dh * sl
-        da = ((dh * b).float() * (sig * (1.0 + a.float() * (1.0 - sig)))).to(torch.bfloat16)
-        dfc1 = torch.cat([da, db], dim=-1)
-        qg, sg, qg_t, sg_t = kernels.tile_quant_dual_grouped(dfc1, goff, E)
+        # through SwiGLU: [da | db] is quantised by the kernel that computes it and never written
+        qg, sg, qg_t, sg_t = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E)
         # through the first linear: dx = dfc1 @ w1 ([M, H]); dw1[n, h] = sum_m dfc1[m, n] x[m, h]
         dx = kernels.grouped_gemm_nt(qg, sg, q1_t, s1_t, goff, out_dtype=x_dtype)
         if ctx.transpose_w1:

@@ -249,6 +249,45 @@ def swiglu_tile_quant_dual_grouped(
     return (q, s, q_t, s_t, h) if return_activation else (q, s, q_t, s_t)
 
 
+def swiglu_bwd_tile_quant_dual_grouped(
+    dh: torch.Tensor,
+    fc1: torch.Tensor,
+    group_offsets: torch.Tensor,
+    num_groups: int,
+    ld_t: Optional[int] = None,
+    rowwise: bool = True,
+    return_grad: bool = False,
+):
+    """Backward of ``h = silu(a) * b`` (rows ``[a | b]`` of ``fc1 [M, 2F]``) for the gradient
+    ``dh [M, F]``, fused into ``tile_quant_dual_grouped`` of the result ``[da | db]``: what autograd
+    makes of SwiGLUActivatition (grouped_gemm_moe.py:331-334) followed by the quantisation of the
+    first grouped linear's output gradient.  Returns ``(q [M,2F], s, q_t [2F, ld_t], s_t)`` (plus
+    the bf16 gradient ``[M, 2F]`` with ``return_grad``)."""
+    assert fc1.dim() == 2 and fc1.is_contiguous() and fc1.dtype == torch.bfloat16
+    assert dh.dim() == 2 and dh.is_contiguous() and dh.dtype == torch.bfloat16
+    M, two_f = fc1.shape
+    assert two_f % (2 * TILE) == 0
+    F = two_f // 2
+    assert dh.shape == (M, F), "dh must be [M, F]"
+    assert group_offsets.dtype == torch.int64 and group_offsets.numel() == num_groups + 1
+    if ld_t is None:
+        ld_t = padded_bound(M, num_groups)
+    dev = fc1.device
+    q = torch.empty((M, two_f), dtype=FP8, device=dev) if rowwise else None
+    s = torch.empty((M, two_f // TILE), dtype=torch.float32, device=dev) if rowwise else None
+    q_t = torch.empty((two_f, ld_t), dtype=FP8, device=dev)
+    s_t = torch.empty((ld_t // TILE, two_f), dtype=torch.float32, device=dev)
+    g = torch.empty((M, two_f), dtype=torch.bfloat16, device=dev) if return_grad else None
+    ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
+    check(
+        lib().aamd_swiglu_bwd_quant_1x128_dual_grouped(
+            ptr(dh), F, ptr(fc1), two_f, M, F, ptr(group_offsets), num_groups, ptr(ws), ptr(g),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, stream(),
+        )
+    )  # fmt: skip
+    return (q, s, q_t, s_t, g) if return_grad else (q, s, q_t, s_t)
+
+
 def block_quant_batched(w: torch.Tensor, eps: float = 0.0, return_transpose: bool = False):
     """128x128 block quantisation of ``w [E, N, K]`` in one launch.
     Returns ``(q [E,N,K], s [E,N/128,K/128], q_t [E,K,N] | None, s_t [E,K/128,N/128] | None)``."""

@@ -131,6 +131,23 @@ int aamd_swiglu_quant_1x128_dual_grouped(const void *fc1, int64_t M, int64_t F, 
                                          uint8_t *q, float *s, uint8_t *q_t, float *s_t, int64_t ld_t, void *stream);
 
 /*
+ * Backward of the gated activation fused into the quantisation of its gradient: for the gradient dh
+ * of h and the saved rows [a | b], the rows [da | db] of d(fc1) are quantised 1x128 row-wise and
+ * transposed inside the ragged groups without being written in bf16.
+ * Replaces what autograd runs for SwiGLUActivatition.forward, atorch/modules/moe/grouped_gemm_moe.py:331-334
+ * (the backward of the multiply, then silu_backward) followed by the per-expert quantize_op.quantize
+ * calls of the first grouped linear's backward, quantized_grouped_linear.py:202-206.
+ *   dh [M, F] bf16 (row stride ld_dh), fc1 [M, 2F] bf16 (row stride ld), F % 128 == 0
+ *   g_out [M, 2F] bf16 or NULL (the gradient itself, for callers that keep it)
+ *   q [M, 2F], s [M, 2F/128] (both may be NULL), q_t [2F, ld_t], s_t [ld_t/128, 2F];
+ *   group_offsets, tile_ws, ld_t as for aamd_quant_1x128_dual_grouped.
+ */
+int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void *dh, int64_t ld_dh, const void *fc1, int64_t ld, int64_t M,
+                                             int64_t F, const int64_t *group_offsets, int E, int32_t *tile_ws,
+                                             void *g_out, uint8_t *q, float *s, uint8_t *q_t, float *s_t,
+                                             int64_t ld_t, void *stream);
+
+/*
  * Ragged grouped block-scaled GEMM, "NT": for every group g and its rows m,
  *   C[m, n] = sum_kb dot(A[m, kb], B_g[n, kb]) * a_s[m, kb] * b_s_g[n/128 or n, kb]  (+ bias_g[n])
  * fp8 x fp8 MFMA, fp32 accumulation, scales applied per 128-deep block.

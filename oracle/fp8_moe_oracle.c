@@ -27,6 +27,7 @@
  *       grouped == per-expert loop, fp64 autograd of the unquantised problem (roles and transposes)
  *   oracle_permute_indices                        pinned: torch.argsort(stable=True), bincount
  *   oracle_swiglu_bf16                            pinned: torch's CPU F.silu and multiply on bf16 tensors
+ *   oracle_swiglu_bwd_bf16                        pinned: torch's CPU autograd of the same two ops, closed forms
  *       (equal except where fp32 silu rounds differently: at most one bf16 ulp, counted in the test),
  *       closed forms silu(0) = 0, silu(x) -> x and -> -0 for large |x|, h == b * silu(a) in double
  *   oracle_unpermute_combine                      pinned: brute force, torch restatement (index_copy_,
@@ -358,6 +359,35 @@ int oracle_swiglu_bf16(const uint16_t *fc1, int64_t rows, int64_t F, int64_t ld,
             const float sl32 = a / (1.0f + e);
             const float sl = bf16_to_f32(f32_to_bf16(sl32));
             h[r * F + c] = f32_to_bf16(sl * b);
+        }
+    return 0;
+}
+
+/*
+ * Backward of the same two torch ops under autograd (grouped_gemm_moe.py:331-334 differentiated:
+ * mul backward, then silu_backward), all tensors bf16:
+ *   db = bf16(dh * bf16(silu(a)))                       grad of the product w.r.t. b: dh * saved silu output
+ *   g  = bf16(dh * b)                                   grad w.r.t. the silu output
+ *   da = bf16(g * sig * (1 + a * (1 - sig))),  sig = 1 / (1 + exp(-a))   silu_backward, fp32 inside,
+ * evaluated left to right as torch's kernel writes it: (g * sig) * (1 + a * (1 - sig)).
+ * dfc1 rows are [da | db] like fc1's [a | b].  Correctly rounded expf as in oracle_swiglu_bf16.
+ */
+int oracle_swiglu_bwd_bf16(const uint16_t *dh, const uint16_t *fc1, int64_t rows, int64_t F, int64_t ld,
+                           uint16_t *dfc1) {
+    if (rows < 0 || F < 0 || ld < 2 * F) return 1;
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < F; c++) {
+            const float a = bf16_to_f32(fc1[r * ld + c]);
+            const float b = bf16_to_f32(fc1[r * ld + F + c]);
+            const float d = bf16_to_f32(dh[r * F + c]);
+            const float e = (float)exp(-(double)a);
+            const float sl = bf16_to_f32(f32_to_bf16(a / (1.0f + e)));
+            const float sig = 1.0f / (1.0f + e);
+            const float g = bf16_to_f32(f32_to_bf16(d * b));
+            const float t = g * sig;
+            const float u = 1.0f + a * (1.0f - sig);
+            dfc1[r * 2 * F + c] = f32_to_bf16(t * u);
+            dfc1[r * 2 * F + F + c] = f32_to_bf16(d * sl);
         }
     return 0;
 }

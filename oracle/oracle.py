@@ -55,6 +55,7 @@ def lib() -> ctypes.CDLL:
         L.oracle_permute_indices.argtypes = [vp, i64, i64, vp, vp]
         L.oracle_unpermute_combine.argtypes = [vp, i64, i64, vp, vp, ci, i64, i64, vp, vp]
         L.oracle_swiglu_bf16.argtypes = [vp, i64, i64, i64, vp]
+        L.oracle_swiglu_bwd_bf16.argtypes = [vp, vp, i64, i64, i64, vp]
         for name in (
             "oracle_tile_quant",
             "oracle_block_quant",
@@ -176,6 +177,18 @@ def swiglu(fc1: torch.Tensor) -> torch.Tensor:
     h = torch.empty((rows, two_f // 2), dtype=torch.int16)
     _chk(lib().oracle_swiglu_bf16(_p(x), rows, two_f // 2, two_f, _p(h)), "swiglu")
     return h.view(torch.bfloat16)
+
+
+def swiglu_bwd(dh: torch.Tensor, fc1: torch.Tensor) -> torch.Tensor:
+    """Gradient of ``swiglu`` w.r.t. ``fc1`` for the output gradient ``dh`` (bf16): rows ``[da | db]``."""
+    assert fc1.dtype == torch.bfloat16 and dh.dtype == torch.bfloat16 and fc1.dim() == 2
+    x = fc1.contiguous().view(torch.int16)
+    d = dh.contiguous().view(torch.int16)
+    rows, two_f = x.shape
+    assert d.shape == (rows, two_f // 2)
+    out = torch.empty((rows, two_f), dtype=torch.int16)
+    _chk(lib().oracle_swiglu_bwd_bf16(_p(d), _p(x), rows, two_f // 2, two_f, _p(out)), "swiglu_bwd")
+    return out.view(torch.bfloat16)
 
 
 def torch_swiglu(fc1: torch.Tensor) -> torch.Tensor:

@@ -79,6 +79,56 @@ def test_swiglu_quant_dual_grouped(oracle, dev, M, F, E):
     assert torch.equal(_u8(q_t3[:, :ptot]), _u8(q_t[:, :ptot])) and torch.equal(s_t3[: ptot // TILE], s_t[: ptot // TILE])
 
 
+def test_swiglu_bwd_over_all_bf16_values(oracle, dev):
+    """[da | db] from the fused backward kernel against the oracle (which equals torch's CPU autograd)
+    for every bf16 value of a below 2^100 in magnitude: hardware exp and reciprocal against correctly
+    rounded ones, so single-ulp differences of the bf16 results on a small fraction of inputs."""
+    from atorch_amd import kernels
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    a = bits[bits.float().abs() < 2.0**100]
+    a = a[: a.numel() // 128 * 128].view(-1, 128)
+    g = torch.Generator().manual_seed(14)
+    b = (torch.randn(a.shape, generator=g) * 2).bfloat16()
+    dh = torch.randn(a.shape, generator=g).bfloat16()
+    fc1 = torch.cat([a, b], dim=1).contiguous()
+    M = fc1.shape[0]
+    goff = kernels.group_offsets_from_splits([M], dev)
+    q, s, q_t, s_t, gr = kernels.swiglu_bwd_tile_quant_dual_grouped(dh.to(dev), fc1.to(dev), goff, 1, return_grad=True)
+    go = oracle.swiglu_bwd(dh, fc1)
+    d = _ulp_diff(gr.cpu(), go)
+    d = torch.where(gr.cpu().float() == go.float(), torch.zeros_like(d), d)
+    assert int(d.max()) <= 1, int(d.max())
+    assert float((d > 0).float().mean()) < 2e-3
+    qo, so = oracle.tile_quant(gr.cpu())
+    assert torch.equal(_u8(q), qo) and torch.equal(s.cpu(), so)
+
+
+@pytest.mark.parametrize("M,F,E", [(300, 256, 3), (1000, 1408 // 128 * 128, 5)])
+def test_swiglu_bwd_quant_dual_grouped(oracle, dev, M, F, E):
+    """The fused backward equals autograd's SwiGLU backward followed by the dual grouped quantisation:
+    outputs bit-identical to tile_quant_dual_grouped of its own gradient, which is within one bf16
+    ulp of the oracle's."""
+    from atorch_amd import kernels
+
+    splits = ragged_splits(M, E, seed=15)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    fc1 = randn_bf16((M, 2 * F), 16, std=2.0)
+    dh = randn_bf16((M, F), 17, std=0.5)
+    q, s, q_t, s_t, gr = kernels.swiglu_bwd_tile_quant_dual_grouped(dh.to(dev), fc1.to(dev), goff, E, return_grad=True)
+    go = oracle.swiglu_bwd(dh, fc1)
+    d = _ulp_diff(gr.cpu(), go)
+    d = torch.where(gr.cpu().float() == go.float(), torch.zeros_like(d), d)
+    assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 2e-3
+    q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(gr, goff, E, ld_t=q_t.shape[1])
+    assert torch.equal(_u8(q), _u8(q2)) and torch.equal(s, s2)
+    ptot = kernels.padded_total(splits)
+    assert torch.equal(s_t[: ptot // TILE], s_t2[: ptot // TILE])
+    assert torch.equal(_u8(q_t[:, :ptot]), _u8(q_t2[:, :ptot]))
+    _, _, q_t3, s_t3 = kernels.swiglu_bwd_tile_quant_dual_grouped(dh.to(dev), fc1.to(dev), goff, E, ld_t=q_t.shape[1], rowwise=False)
+    assert torch.equal(_u8(q_t3[:, :ptot]), _u8(q_t[:, :ptot])) and torch.equal(s_t3[: ptot // TILE], s_t[: ptot // TILE])
+
+
 def test_swiglu_quant_rejects_bad_shapes(dev):
     from atorch_amd import kernels
 
