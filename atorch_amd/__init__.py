@@ -10,6 +10,7 @@ that mirrors the reference's Python surfaces for this path:
 * ``atorch_amd.token_dispatcher`` - ``permute`` / ``unpermute`` and the single-GPU dispatcher;
 * ``atorch_amd.gmm``              - the ``gmm(a, b, batch_sizes, trans_b)`` adapter;
 * ``atorch_amd.expert_mlp``       - ``gmm -> SwiGLU -> gmm`` of an expert MLP, SwiGLU fused into the quantiser;
+* ``atorch_amd.bias_gather_add``  - per-expert bias on expert-tagged rows and its bias gradient;
 * ``atorch_amd.ops``              - the module the reference's dense FP8 wrappers load by name.
 """
 __version__ = "0.1.0"

@@ -39,6 +39,8 @@ SIGNATURES = {
         _int,
         [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
     ),
+    "aamd_bias_gather_add": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
+    "aamd_bias_gather_add_bgrad": (_int, [_vp, _vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
     "aamd_quant_128x128": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp]),
     "aamd_dequant": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _int, _vp]),
     "aamd_grouped_gemm_fp8_nt": (

@@ -252,9 +252,151 @@ __global__ __launch_bounds__(256) void route_place_kernel(const ID* __restrict__
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Per-expert bias on expert-tagged rows: out[t] = inp[t] + bias[bin_ids[t]] and its bias gradient
+// ---------------------------------------------------------------------------------------
+template <typename ID>
+__global__ __launch_bounds__(256) void bias_gather_add_kernel(const v4i* __restrict__ inp, const v4i* __restrict__ bias,
+                                                              const ID* __restrict__ bin_ids, int64_t chunks, int row_chunks,
+                                                              int E, bool is_bf16, v4i* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= chunks) return;
+  const int64_t t = i / row_chunks;
+  const int c = (int)(i - t * row_chunks);
+  const int64_t e = (int64_t)bin_ids[t];
+  const v4i a = __builtin_nontemporal_load(inp + i);
+  v4i r = a;
+  if (e >= 0 && e < E) {
+    const v4i b = bias[e * row_chunks + c];
+    if (is_bf16) {
+      float fa[8], fb[8];
+      unpack8(a, fa);
+      unpack8(b, fb);
+#pragma unroll
+      for (int k = 0; k < 4; k++) r[k] = (int)pack_bf16x2(fa[2 * k] + fb[2 * k], fa[2 * k + 1] + fb[2 * k + 1]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; k++) r[k] = __float_as_int(__int_as_float(a[k]) + __int_as_float(b[k]));
+    }
+  }
+  __builtin_nontemporal_store(r, out + i);
+}
+
+__global__ __launch_bounds__(256) void fill_zero_f32_kernel(float* __restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+// bgrad[e, :] += sum of the rows tagged e.  A workgroup walks kBgRows consecutive rows; a thread owns
+// one 16-byte chunk of columns and keeps the running sum of the current expert in registers, so rows
+// grouped by expert cost one set of atomics per workgroup and expert.
+constexpr int kBgRows = 128;
+template <typename ID>
+__global__ __launch_bounds__(256) void bias_gather_bgrad_kernel(const v4i* __restrict__ grad, const ID* __restrict__ bin_ids,
+                                                                int64_t T, int row_chunks, int E, bool is_bf16,
+                                                                float* __restrict__ bgrad) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= row_chunks) return;
+  const int64_t t0 = (int64_t)blockIdx.y * kBgRows;
+  const int64_t t1 = t0 + kBgRows < T ? t0 + kBgRows : T;
+  const int W = is_bf16 ? 8 : 4;  // columns per chunk
+  float acc[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) acc[k] = 0.f;
+  int64_t cur = -1;
+  auto flush = [&]() {
+    if (cur < 0 || cur >= E) return;
+    float* dst = bgrad + cur * (int64_t)row_chunks * W + (int64_t)c * W;
+    for (int k = 0; k < W; k++) atomicAdd(dst + k, acc[k]);
+  };
+  constexpr int B = 8;  // rows in flight per thread
+  for (int64_t tb = t0; tb < t1; tb += B) {
+    v4i g[B];
+    int64_t e[B];
+#pragma unroll
+    for (int u = 0; u < B; u++) {
+      const int64_t t = tb + u < t1 ? tb + u : t1 - 1;
+      e[u] = tb + u < t1 ? (int64_t)bin_ids[t] : -2;  // -2: past the end, skipped below
+      g[u] = __builtin_nontemporal_load(grad + t * row_chunks + c);
+    }
+#pragma unroll
+    for (int u = 0; u < B; u++) {
+      if (e[u] == -2) continue;
+      if (e[u] != cur) {
+        flush();
+#pragma unroll
+        for (int k = 0; k < 8; k++) acc[k] = 0.f;
+        cur = e[u];
+      }
+      if (is_bf16) {
+        float f[8];
+        unpack8(g[u], f);
+#pragma unroll
+        for (int k = 0; k < 8; k++) acc[k] += f[k];
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; k++) acc[k] += __int_as_float(g[u][k]);
+      }
+    }
+  }
+  flush();
+}
+
 }  // namespace aamd
 
 using namespace aamd;
+
+extern "C" int aamd_bias_gather_add(const void* inp, const void* bias, const void* bin_ids, int ids_are_i64, int64_t T,
+                                    int64_t H, int E, int dtype, void* out, void* stream) {
+  AAMD_REQUIRE(dtype == AAMD_BF16 || dtype == AAMD_F32, "bias_gather_add: unsupported dtype %d", dtype);
+  const int64_t row_bytes = H * (dtype == AAMD_BF16 ? 2 : 4);
+  AAMD_REQUIRE(T >= 0 && H >= 0 && E >= 1 && row_bytes % 16 == 0, "bias_gather_add: row size must be a multiple of 16 bytes");
+  if (T == 0 || H == 0) return AAMD_OK;
+  AAMD_REQUIRE(inp && bias && bin_ids && out, "bias_gather_add: null pointer");
+  AAMD_REQUIRE(((uintptr_t)inp & 15) == 0 && ((uintptr_t)bias & 15) == 0 && ((uintptr_t)out & 15) == 0,
+               "bias_gather_add: pointers must be 16-byte aligned");
+  const int64_t rc = row_bytes / 16, chunks = T * rc;
+  AAMD_REQUIRE(rc < 0x7fffffffLL && (chunks + 255) / 256 < 0x7fffffffLL, "bias_gather_add: too large");
+  const unsigned blocks = (unsigned)((chunks + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+  if (ids_are_i64)
+    bias_gather_add_kernel<int64_t><<<blocks, 256, 0, st>>>((const v4i*)inp, (const v4i*)bias, (const int64_t*)bin_ids, chunks,
+                                                            (int)rc, E, dtype == AAMD_BF16, (v4i*)out);
+  else
+    bias_gather_add_kernel<int32_t><<<blocks, 256, 0, st>>>((const v4i*)inp, (const v4i*)bias, (const int32_t*)bin_ids, chunks,
+                                                            (int)rc, E, dtype == AAMD_BF16, (v4i*)out);
+  AAMD_LAUNCH_CHECK("bias_gather_add");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_bias_gather_add_bgrad(const void* grad, const void* bin_ids, int ids_are_i64, int64_t T, int64_t H,
+                                          int E, int dtype, float* bgrad, void* stream) {
+  AAMD_REQUIRE(dtype == AAMD_BF16 || dtype == AAMD_F32, "bias_gather_add_bgrad: unsupported dtype %d", dtype);
+  const int64_t row_bytes = H * (dtype == AAMD_BF16 ? 2 : 4);
+  AAMD_REQUIRE(T >= 0 && H >= 0 && E >= 1 && row_bytes % 16 == 0,
+               "bias_gather_add_bgrad: row size must be a multiple of 16 bytes");
+  if (H == 0) return AAMD_OK;
+  AAMD_REQUIRE(bgrad != nullptr, "bias_gather_add_bgrad: null output");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = (int64_t)E * H;
+  AAMD_REQUIRE((n + 255) / 256 < 0x7fffffffLL, "bias_gather_add_bgrad: too large");
+  fill_zero_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(bgrad, n);  // a kernel, so callers may capture it
+  AAMD_LAUNCH_CHECK("bias_gather_add_bgrad (clear)");
+  if (T == 0) return AAMD_OK;
+  AAMD_REQUIRE(grad && bin_ids, "bias_gather_add_bgrad: null pointer");
+  AAMD_REQUIRE(((uintptr_t)grad & 15) == 0, "bias_gather_add_bgrad: grad must be 16-byte aligned");
+  const int64_t rc = row_bytes / 16, row_blocks = (T + kBgRows - 1) / kBgRows;
+  AAMD_REQUIRE(rc < 0x7fffffffLL && row_blocks <= 65535, "bias_gather_add_bgrad: more than 65535 * 128 rows");
+  dim3 grid((unsigned)((rc + 255) / 256), (unsigned)row_blocks), block(256);
+  if (ids_are_i64)
+    bias_gather_bgrad_kernel<int64_t><<<grid, block, 0, st>>>((const v4i*)grad, (const int64_t*)bin_ids, T, (int)rc, E,
+                                                              dtype == AAMD_BF16, bgrad);
+  else
+    bias_gather_bgrad_kernel<int32_t><<<grid, block, 0, st>>>((const v4i*)grad, (const int32_t*)bin_ids, T, (int)rc, E,
+                                                              dtype == AAMD_BF16, bgrad);
+  AAMD_LAUNCH_CHECK("bias_gather_add_bgrad");
+  return AAMD_OK;
+}
 
 extern "C" int aamd_unpermute_combine(const void* y, int64_t M, int64_t H, const int32_t* row_map,
                                       const void* probs, int probs_dtype, int64_t T, int topk, void* out,

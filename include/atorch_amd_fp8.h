@@ -215,6 +215,22 @@ int aamd_moe_preprocess(const void *expert_ids, int ids_are_i64, int64_t n, int 
 int aamd_invert_permutation(const int64_t *sorted_idx, int64_t n_perm, int64_t n_flat, int32_t *row_map,
                             void *stream);
 
+/*
+ * Per-expert bias on rows tagged with their expert: out[t, :] = inp[t, :] + bias[bin_ids[t], :]
+ * (bf16: the fp32 sum rounded to bf16), and its bias gradient bgrad[e, :] = sum of grad[t, :] over
+ * the rows with bin_ids[t] == e, accumulated in fp32 (order of the additions unspecified, as with
+ * the reference's atomic adds; the caller casts to the gradient's dtype).
+ * Replaces bias_gather_add_fw / bias_gather_add_bw, atorch/kernels/triton_jit/bias_gather_add.py:50-66, 101-127.
+ *   inp, out, grad [T, H] and bias [E, H] of `dtype`; H * sizeof(dtype) % 16 == 0
+ *   bin_ids [T]: int64 when ids_are_i64 != 0, else int32; rows tagged outside [0, E) pass through
+ *   unchanged and add nothing to bgrad
+ *   bgrad [E, H] fp32, cleared by the call.
+ */
+int aamd_bias_gather_add(const void *inp, const void *bias, const void *bin_ids, int ids_are_i64, int64_t T,
+                         int64_t H, int E, int dtype, void *out, void *stream);
+int aamd_bias_gather_add_bgrad(const void *grad, const void *bin_ids, int ids_are_i64, int64_t T, int64_t H, int E,
+                               int dtype, float *bgrad, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

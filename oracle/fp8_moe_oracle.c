@@ -27,6 +27,7 @@
  *       grouped == per-expert loop, fp64 autograd of the unquantised problem (roles and transposes)
  *   oracle_permute_indices                        pinned: torch.argsort(stable=True), bincount
  *   oracle_swiglu_bf16                            pinned: torch's CPU F.silu and multiply on bf16 tensors
+ *   oracle_bias_gather_add / _bgrad               pinned: torch index and index_add_ on the CPU, exact-sum data
  *   oracle_swiglu_bwd_bf16                        pinned: torch's CPU autograd of the same two ops, closed forms
  *       (equal except where fp32 silu rounds differently: at most one bf16 ulp, counted in the test),
  *       closed forms silu(0) = 0, silu(x) -> x and -> -0 for large |x|, h == b * silu(a) in double
@@ -338,6 +339,46 @@ int oracle_unpermute_combine(const uint16_t *y, int64_t n_perm, int64_t H, const
                 out_bf16[t * H + h] = f32_to_bf16(acc);
         }
     free(inv);
+    return 0;
+}
+
+/*
+ * Per-expert bias on expert-tagged rows, atorch/kernels/triton_jit/bias_gather_add.py:24-47 (forward:
+ * out[t] = inp[t] + bias[bin_ids[t]], in the tensors' dtype: a bf16 sum is the fp32 sum rounded) and
+ * :80-98 (backward: bgrad[e] = fp32 sum of the rows tagged e; the reference adds atomically in no
+ * fixed order, here in row order).  is_bf16 selects bf16 bit patterns or fp32 for inp / bias / out / grad.
+ */
+int oracle_bias_gather_add(const void *inp, const void *bias, const int64_t *bin_ids, int64_t T, int64_t H, int E,
+                           int is_bf16, void *out) {
+    if (T < 0 || H < 0 || E < 1) return 1;
+    for (int64_t t = 0; t < T; t++) {
+        const int64_t e = bin_ids[t];
+        if (e < 0 || e >= E) return 2;
+        for (int64_t c = 0; c < H; c++) {
+            if (is_bf16) {
+                const float a = bf16_to_f32(((const uint16_t *)inp)[t * H + c]);
+                const float b = bf16_to_f32(((const uint16_t *)bias)[e * H + c]);
+                ((uint16_t *)out)[t * H + c] = f32_to_bf16(a + b);
+            } else {
+                ((float *)out)[t * H + c] = ((const float *)inp)[t * H + c] + ((const float *)bias)[e * H + c];
+            }
+        }
+    }
+    return 0;
+}
+
+int oracle_bias_gather_bgrad(const void *grad, const int64_t *bin_ids, int64_t T, int64_t H, int E, int is_bf16,
+                             float *bgrad) {
+    if (T < 0 || H < 0 || E < 1) return 1;
+    for (int64_t i = 0; i < (int64_t)E * H; i++) bgrad[i] = 0.0f;
+    for (int64_t t = 0; t < T; t++) {
+        const int64_t e = bin_ids[t];
+        if (e < 0 || e >= E) return 2;
+        for (int64_t c = 0; c < H; c++) {
+            const float g = is_bf16 ? bf16_to_f32(((const uint16_t *)grad)[t * H + c]) : ((const float *)grad)[t * H + c];
+            bgrad[e * H + c] += g;
+        }
+    }
     return 0;
 }
 

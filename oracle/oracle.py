@@ -56,6 +56,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_unpermute_combine.argtypes = [vp, i64, i64, vp, vp, ci, i64, i64, vp, vp]
         L.oracle_swiglu_bf16.argtypes = [vp, i64, i64, i64, vp]
         L.oracle_swiglu_bwd_bf16.argtypes = [vp, vp, i64, i64, i64, vp]
+        L.oracle_bias_gather_add.argtypes = [vp, vp, vp, i64, i64, ci, ci, vp]
+        L.oracle_bias_gather_bgrad.argtypes = [vp, vp, i64, i64, ci, ci, vp]
         for name in (
             "oracle_tile_quant",
             "oracle_block_quant",
@@ -189,6 +191,30 @@ def swiglu_bwd(dh: torch.Tensor, fc1: torch.Tensor) -> torch.Tensor:
     out = torch.empty((rows, two_f), dtype=torch.int16)
     _chk(lib().oracle_swiglu_bwd_bf16(_p(d), _p(x), rows, two_f // 2, two_f, _p(out)), "swiglu_bwd")
     return out.view(torch.bfloat16)
+
+
+def bias_gather_add(inp: torch.Tensor, bias: torch.Tensor, bin_ids: torch.Tensor) -> torch.Tensor:
+    """bias_gather_add.py:50-66: ``inp + bias[bin_ids]`` in the tensors' dtype (bf16 or fp32)."""
+    assert inp.dtype == bias.dtype and inp.dtype in (torch.bfloat16, torch.float32)
+    bf = inp.dtype == torch.bfloat16
+    a = inp.contiguous().view(torch.int16) if bf else inp.contiguous()
+    b = bias.contiguous().view(torch.int16) if bf else bias.contiguous()
+    ids = bin_ids.to(torch.int64).contiguous()
+    out = torch.empty_like(a)
+    T, H = a.shape
+    _chk(lib().oracle_bias_gather_add(_p(a), _p(b), _p(ids), T, H, bias.shape[0], int(bf), _p(out)), "bias_gather_add")
+    return out.view(torch.bfloat16) if bf else out
+
+
+def bias_gather_bgrad(grad: torch.Tensor, bin_ids: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """bias_gather_add.py:101-127: fp32 sums of the rows of each expert (row order), ``[E, H]`` fp32."""
+    bf = grad.dtype == torch.bfloat16
+    g = grad.contiguous().view(torch.int16) if bf else grad.contiguous()
+    ids = bin_ids.to(torch.int64).contiguous()
+    T, H = g.shape
+    out = torch.empty((num_experts, H), dtype=torch.float32)
+    _chk(lib().oracle_bias_gather_bgrad(_p(g), _p(ids), T, H, num_experts, int(bf), _p(out)), "bias_gather_bgrad")
+    return out
 
 
 def torch_swiglu(fc1: torch.Tensor) -> torch.Tensor:

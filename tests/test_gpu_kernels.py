@@ -499,3 +499,53 @@ def test_grouped_gemm_wgrad(oracle, dev, M, N, K, E, mult):
     for e, m in enumerate(splits):
         if m == 0:
             assert torch.equal(acc[e].cpu(), base[e])
+
+
+# ------------------------------------------------------------------------------------------
+# f4: per-expert bias on expert-tagged rows
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("ids_dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("T,H,E", [(1, 8, 1), (300, 136, 5), (4097, 1024, 64)])
+def test_bias_gather_add_matches_oracle(oracle, dev, dtype, ids_dtype, T, H, E):
+    from atorch_amd.bias_gather_add import bias_gather_add_bw, bias_gather_add_fw
+
+    g = torch.Generator().manual_seed(T + H)
+    ids = torch.randint(0, E, (T,), generator=g).sort().values  # grouped by expert, as the dispatcher leaves them
+    inp = torch.randn(T, H, generator=g).to(dtype)
+    bias = torch.randn(E, H, generator=g).to(dtype)
+    out = bias_gather_add_fw(inp.to(dev), bias.to(dev), ids.to(ids_dtype).to(dev))
+    assert torch.equal(out.cpu().view(torch.uint8), oracle.bias_gather_add(inp, bias, ids).view(torch.uint8))
+    # sums that are exact in fp32: any order of additions gives the same bits
+    small = torch.randint(-8, 9, (T, H), generator=g).to(dtype)
+    bg = bias_gather_add_bw(small.to(dev), ids.to(ids_dtype).to(dev), E)
+    assert bg.dtype == dtype
+    assert torch.equal(bg.cpu().float(), oracle.bias_gather_bgrad(small, ids, E).to(dtype).float())
+    # random data and unsorted tags: fp32 sums in another order, compared in fp32 before the final cast
+    ids_u = ids[torch.randperm(T, generator=g)]
+    bg2 = bias_gather_add_bw(inp.float().to(dev), ids_u.to(ids_dtype).to(dev), E)
+    ref = oracle.bias_gather_bgrad(inp.float(), ids_u, E)
+    assert float((bg2.cpu() - ref).abs().max()) <= 1e-5 * max(1.0, float(ref.abs().max()))
+
+
+def test_bias_gather_add_autograd_and_edges(oracle, dev):
+    from atorch_amd.bias_gather_add import bias_gather_add, bias_gather_add_bw, bias_gather_add_fw
+
+    g = torch.Generator().manual_seed(8)
+    T, H, E = 515, 256, 6
+    ids = torch.randint(0, E, (T,), generator=g).sort().values.to(dev)
+    inp = torch.randn(T, H, generator=g).bfloat16().to(dev).requires_grad_(True)
+    bias = torch.randn(E, H, generator=g).bfloat16().to(dev).requires_grad_(True)
+    dy = torch.randint(-4, 5, (T, H), generator=g).bfloat16().to(dev)
+    bias_gather_add(inp, bias, ids).backward(dy)
+    assert torch.equal(inp.grad, dy)
+    assert torch.equal(bias.grad.cpu().float(), oracle.bias_gather_bgrad(dy.cpu(), ids.cpu(), E).bfloat16().float())
+    # no rows: empty output, zero gradient
+    z = bias_gather_add_fw(torch.empty(0, H, dtype=torch.bfloat16, device=dev), bias.detach(), torch.empty(0, dtype=torch.int64, device=dev))
+    assert z.shape == (0, H)
+    zb = bias_gather_add_bw(torch.empty(0, H, dtype=torch.bfloat16, device=dev), torch.empty(0, dtype=torch.int64, device=dev), E)
+    assert zb.shape == (E, H) and float(zb.abs().max()) == 0.0
+    with pytest.raises(ValueError):
+        bias_gather_add_fw(torch.zeros(4, 12, dtype=torch.bfloat16, device=dev), torch.zeros(2, 12, dtype=torch.bfloat16, device=dev),
+                           torch.zeros(4, dtype=torch.int64, device=dev))  # 24-byte rows
+
