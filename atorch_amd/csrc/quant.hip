@@ -38,6 +38,22 @@ struct Raw8<F32> {
   }
 };
 
+// sigmoid on the hardware transcendental units, one v_exp_f32 and one v_rcp_f32 per value.  Both
+// flush results below the normal range, and 1 / (1 + e^-x) gets there for x below about -87 while
+// x times it is still a normal number, so everything is carried scaled by 2^16 (x r' stays finite for
+// |x| < 2^112):
+//   e' = 2^-16 e^-x (inf where e^-x itself overflows), r' = 1 / (2^-16 + e') = 2^16 sigmoid(x).
+// silu(x) = (x r') 2^-16, sigmoid(x) = r' 2^-16.  A few fp32 ulps of error (more for |x| in the tens,
+// where x log2(e) itself is rounded), far below the bf16 rounding that follows; e^-x = inf gives
+// r' = 0 and silu = -0 as in fp32 arithmetic.
+__device__ __forceinline__ float sigmoid_scaled(float x) {
+  const float t = x * -1.4426950408889634f;
+  float e = __builtin_amdgcn_exp2f(t - 16.0f);
+  e = t >= 128.0f ? __builtin_inff() : e;  // where e^-x overflows in fp32 it does so here too
+  return __builtin_amdgcn_rcpf(0x1p-16f + e);
+}
+__device__ __forceinline__ float silu_from(float x, float r_scaled) { return (x * r_scaled) * 0x1p-16f; }
+
 // SwiGLU on load: a and b halves of a row, h = silu(a) * b with both roundings to bf16 that the
 // reference's two torch ops make (F.silu on a bf16 tensor, then the product; fp32 inside).
 template <>
@@ -54,9 +70,8 @@ struct Raw8<GLU> {
     unpack8(b, fb);
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
-      // hardware exp2 and reciprocal: a few fp32 ulps, far below the bf16 rounding that follows
-      const float s0 = __fdividef(fa[i], 1.0f + __expf(-fa[i]));
-      const float s1 = __fdividef(fa[i + 1], 1.0f + __expf(-fa[i + 1]));
+      const float s0 = silu_from(fa[i], sigmoid_scaled(fa[i]));
+      const float s1 = silu_from(fa[i + 1], sigmoid_scaled(fa[i + 1]));
       const uint32_t sl = pack_bf16x2(s0, s1);
       const uint32_t h = pack_bf16x2(__uint_as_float(sl << 16) * fb[i], __uint_as_float(sl & 0xffff0000u) * fb[i + 1]);
       v[i] = __uint_as_float(h << 16);
@@ -70,8 +85,8 @@ struct Raw8<GLU> {
 struct GluBwd8 {
   v4i a, b, d;
   __device__ __forceinline__ void load(const u16* pa, int64_t gate_off, const u16* pd, bool want_db) {
-    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pa));
-    d = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pd));
+    a = *reinterpret_cast<const v4i*>(pa);  // a and dh are read by both teams: plain loads, kept in the caches
+    d = *reinterpret_cast<const v4i*>(pd);
     if (!want_db) b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pa + gate_off));
     else b = v4i{0, 0, 0, 0};
   }
@@ -84,14 +99,13 @@ struct GluBwd8 {
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
       float r0, r1;
-      // hardware exp2 and reciprocal, as in the forward loader
-      const float e0 = __expf(-fa[i]), e1 = __expf(-fa[i + 1]);
+      const float rs0 = sigmoid_scaled(fa[i]), rs1 = sigmoid_scaled(fa[i + 1]);
       if (want_db) {
-        const uint32_t sl = pack_bf16x2(__fdividef(fa[i], 1.0f + e0), __fdividef(fa[i + 1], 1.0f + e1));
+        const uint32_t sl = pack_bf16x2(silu_from(fa[i], rs0), silu_from(fa[i + 1], rs1));
         r0 = fd[i] * __uint_as_float(sl << 16);
         r1 = fd[i + 1] * __uint_as_float(sl & 0xffff0000u);
       } else {
-        const float sg0 = __fdividef(1.0f, 1.0f + e0), sg1 = __fdividef(1.0f, 1.0f + e1);
+        const float sg0 = rs0 * 0x1p-16f, sg1 = rs1 * 0x1p-16f;
         const uint32_t g = pack_bf16x2(fd[i] * fb[i], fd[i + 1] * fb[i + 1]);
         r0 = (__uint_as_float(g << 16) * sg0) * (1.0f + fa[i] * (1.0f - sg0));
         r1 = (__uint_as_float(g & 0xffff0000u) * sg1) * (1.0f + fa[i + 1] * (1.0f - sg1));
@@ -177,11 +191,13 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
 // 256 threads, thread (gr = tid/16, c = tid%16) holds rows gr*8 .. gr*8+7, columns c*8 .. c*8+7.
 // ---------------------------------------------------------------------------------------
 constexpr int kTLd = kTile + 16;  // LDS row stride (bytes) of the transposed code tile
+// thread index inside a 256-thread tile team (a workgroup is one team, or two for the SwiGLU backward)
+__device__ __forceinline__ int team_tid() { return threadIdx.x & 255; }
 
 template <typename IN>
 __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, int64_t ldx, int rows_valid,
                                           float (&v)[8][8], int64_t gate_off = 0) {
-  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+  const int gr = team_tid() >> 4, c = team_tid() & 15;
   Raw8<IN> raw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
@@ -199,7 +215,7 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
 __device__ __forceinline__ void load_tile_glu_bwd(const u16* __restrict__ fc1, int64_t ld, int64_t gate_off,
                                                   const u16* __restrict__ dh, int64_t ld_dh, bool want_db,
                                                   int rows_valid, float (&v)[8][8]) {
-  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+  const int gr = team_tid() >> 4, c = team_tid() & 15;
   GluBwd8 raw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
@@ -218,7 +234,7 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
   __syncthreads();
 #pragma unroll
   for (int n = 0; n < 4; n++) {
-    const int idx = threadIdx.x + 256 * n;
+    const int idx = team_tid() + 256 * n;
     const int r = idx >> 3, ch = idx & 7;
     __builtin_nontemporal_store(*reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16),
                                 reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16));
@@ -229,7 +245,7 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
 // out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
 __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const float* cs, uint8_t* tile_t,
                                                  uint8_t* __restrict__ out, int64_t ld_out, bool plain_div) {
-  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+  const int gr = team_tid() >> 4, c = team_tid() & 15;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
     float col[8];
@@ -241,33 +257,36 @@ __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const f
 }
 
 template <typename IN>
-__global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
+__global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void quant_dual_grouped_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
     u16* __restrict__ h_out, const u16* __restrict__ dh = nullptr, int64_t ld_dh = 0) {
   const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
-  __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
-  static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_t), "the column maxima fit in the staging region");
+  // SwiGLU backward: two teams of 256 threads per workgroup, one for the da tile and one for the db
+  // tile of the same features, each with its own staging; both read a and dh at the same time, so
+  // the second read is served by the caches and HBM sees every input once
+  constexpr int TEAMS = std::is_same<IN, GLUB>::value ? 2 : 1;
+  const int team = TEAMS == 2 ? (int)(threadIdx.x >> 8) : 0;
+  __shared__ __attribute__((aligned(16))) uint8_t tile_ts[TEAMS][kTile * kTLd];
+  static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_ts[0]), "the column maxima fit in the staging region");
+  uint8_t* const tile_t = tile_ts[team];
   float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
-  __shared__ float cscale[kTile];
+  __shared__ float cscales[TEAMS][kTile];
+  float* const cscale = cscales[team];
   __shared__ int slot;
 
   int kc = blockIdx.x;
   const int pt = blockIdx.y;
-  if constexpr (std::is_same<IN, GLUB>::value) {
-    // consecutive workgroups take the da and the db tile of the same features: the second one finds
-    // a and dh in the L2
-    kc = (blockIdx.x & 1) * (nt / 2) + (blockIdx.x >> 1);
-  }
+  if constexpr (TEAMS == 2) kc = team * (nt / 2) + blockIdx.x;  // da tiles first, then db tiles
   const int g = find_group(tile_off, E, pt, &slot);
   if (g >= E) return;
   const int64_t cols = (int64_t)nt * kTile;
   const int64_t m0 = goff[g] + (int64_t)(pt - tile_off[g]) * kTile;
   const int64_t left = goff[g + 1] - m0;
   const int mvalid = left < kTile ? (int)left : kTile;
-  const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
+  const int gr = team_tid() >> 4, c = team_tid() & 15;
 
   float v[8][8];
   if constexpr (std::is_same<IN, GLUB>::value) {
@@ -303,13 +322,13 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
 #pragma unroll
   for (int j = 0; j < 8; j++) part[gr][c * 8 + j] = cm[j];
   __syncthreads();
-  if (threadIdx.x < kTile) {
-    float m = part[0][threadIdx.x];
+  if (team_tid() < kTile) {
+    float m = part[0][team_tid()];
 #pragma unroll
-    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][threadIdx.x]);
+    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][team_tid()]);
     const float sc = scale_from_amax(m, eps);
-    cscale[threadIdx.x] = sc;
-    s_t[(int64_t)pt * cols + (int64_t)kc * kTile + threadIdx.x] = sc;
+    cscale[team_tid()] = sc;
+    s_t[(int64_t)pt * cols + (int64_t)kc * kTile + team_tid()] = sc;
   }
   __syncthreads();
   float cs[8];
@@ -613,7 +632,7 @@ extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t 
   int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
   if (rc) return rc;
   const int nt = (int)(2 * F / kTile);
-  dim3 grid((unsigned)nt, (unsigned)grid_tiles), block(256);
+  dim3 grid((unsigned)(nt / 2), (unsigned)grid_tiles), block(512);  // two teams: the da and the db tile of a feature tile
   quant_dual_grouped_kernel<GLUB><<<grid, block, 0, st>>>((const u16*)fc1, ld, nt, group_offsets, tile_ws, E, q, s, q_t, s_t,
                                                           ld_t, 0.f, F, (u16*)g_out, (const u16*)dh, ld_dh);
   AAMD_LAUNCH_CHECK("swiglu_bwd_quant_dual_grouped");

@@ -31,8 +31,9 @@ def _ulp_diff(a, b):
 
 def test_swiglu_over_all_bf16_values(oracle, dev):
     """h from the fused kernel against the oracle for every finite bf16 value of a: the kernel
-    evaluates silu in fp32 (x / (1 + expf(-x))), the oracle rounds the exact value, so single-ulp
-    differences of the bf16 result are allowed on a small fraction of inputs; nothing larger."""
+    evaluates sigmoid with the hardware exp2 and reciprocal (a few fp32 ulps), the oracle with a
+    correctly rounded expf, so bf16(silu) may differ by one ulp on a small fraction of inputs; the
+    product with b is rounded again, which can turn that into two ulps of h, never more."""
     from atorch_amd import kernels
 
     bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
@@ -46,7 +47,7 @@ def test_swiglu_over_all_bf16_values(oracle, dev):
     d = _ulp_diff(h.cpu(), ho)
     # +-0 differ by 0x8000 as integers but are equal values
     d = torch.where(h.cpu().float() == ho.float(), torch.zeros_like(d), d)
-    assert int(d.max()) <= 1, int(d.max())
+    assert int(d.max()) <= 2, int(d.max())
     assert float((d > 0).float().mean()) < 2e-3
     # the codes and scales are exactly the quantisation of the kernel's own activation
     qo, so = oracle.tile_quant(h.cpu())
@@ -57,7 +58,7 @@ def test_swiglu_over_all_bf16_values(oracle, dev):
 def test_swiglu_quant_dual_grouped(oracle, dev, M, F, E):
     """The fused kernel equals SwiGLU followed by the dual (row + transposed) grouped quantisation:
     its outputs are bit-identical to tile_quant_dual_grouped applied to its own activation, which
-    is within one bf16 ulp of the oracle's."""
+    is within two bf16 ulps of the oracle's (one for bf16(silu), rounded again in the product)."""
     from atorch_amd import kernels
 
     splits = ragged_splits(M, E, seed=5)
@@ -67,7 +68,7 @@ def test_swiglu_quant_dual_grouped(oracle, dev, M, F, E):
     ho = oracle.swiglu(fc1)
     d = _ulp_diff(h.cpu(), ho)
     d = torch.where(h.cpu().float() == ho.float(), torch.zeros_like(d), d)
-    assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 2e-3
+    assert int(d.max()) <= 2 and float((d > 0).float().mean()) < 2e-3
     q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(h, goff, E, ld_t=q_t.shape[1])
     assert torch.equal(_u8(q), _u8(q2)) and torch.equal(s, s2)
     # columns / scale rows past the padded total are not written by either kernel
@@ -82,7 +83,8 @@ def test_swiglu_quant_dual_grouped(oracle, dev, M, F, E):
 def test_swiglu_bwd_over_all_bf16_values(oracle, dev):
     """[da | db] from the fused backward kernel against the oracle (which equals torch's CPU autograd)
     for every bf16 value of a below 2^100 in magnitude: hardware exp and reciprocal against correctly
-    rounded ones, so single-ulp differences of the bf16 results on a small fraction of inputs."""
+    rounded ones, so differences of one bf16 ulp (two in db, whose bf16(silu) factor is rounded
+    again in the product) on a small fraction of inputs."""
     from atorch_amd import kernels
 
     bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
@@ -98,7 +100,7 @@ def test_swiglu_bwd_over_all_bf16_values(oracle, dev):
     go = oracle.swiglu_bwd(dh, fc1)
     d = _ulp_diff(gr.cpu(), go)
     d = torch.where(gr.cpu().float() == go.float(), torch.zeros_like(d), d)
-    assert int(d.max()) <= 1, int(d.max())
+    assert int(d.max()) <= 2, int(d.max())
     assert float((d > 0).float().mean()) < 2e-3
     qo, so = oracle.tile_quant(gr.cpu())
     assert torch.equal(_u8(q), qo) and torch.equal(s.cpu(), so)
@@ -107,8 +109,8 @@ def test_swiglu_bwd_over_all_bf16_values(oracle, dev):
 @pytest.mark.parametrize("M,F,E", [(300, 256, 3), (1000, 1408 // 128 * 128, 5)])
 def test_swiglu_bwd_quant_dual_grouped(oracle, dev, M, F, E):
     """The fused backward equals autograd's SwiGLU backward followed by the dual grouped quantisation:
-    outputs bit-identical to tile_quant_dual_grouped of its own gradient, which is within one bf16
-    ulp of the oracle's."""
+    outputs bit-identical to tile_quant_dual_grouped of its own gradient, which is within two bf16
+    ulps of the oracle's."""
     from atorch_amd import kernels
 
     splits = ragged_splits(M, E, seed=15)
@@ -119,7 +121,7 @@ def test_swiglu_bwd_quant_dual_grouped(oracle, dev, M, F, E):
     go = oracle.swiglu_bwd(dh, fc1)
     d = _ulp_diff(gr.cpu(), go)
     d = torch.where(gr.cpu().float() == go.float(), torch.zeros_like(d), d)
-    assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 2e-3
+    assert int(d.max()) <= 2 and float((d > 0).float().mean()) < 2e-3
     q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(gr, goff, E, ld_t=q_t.shape[1])
     assert torch.equal(_u8(q), _u8(q2)) and torch.equal(s, s2)
     ptot = kernels.padded_total(splits)
