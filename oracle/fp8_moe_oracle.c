@@ -26,11 +26,13 @@
  *       pure-Python brute force in the reference's accumulation order, linearity / accumulate,
  *       grouped == per-expert loop, fp64 autograd of the unquantised problem (roles and transposes)
  *   oracle_permute_indices                        pinned: torch.argsort(stable=True), bincount
- *   oracle_swiglu_bf16                            pinned: torch's CPU F.silu and multiply on bf16 tensors
- *   oracle_bias_gather_add / _bgrad               pinned: torch index and index_add_ on the CPU, exact-sum data
- *   oracle_swiglu_bwd_bf16                        pinned: torch's CPU autograd of the same two ops, closed forms
- *       (equal except where fp32 silu rounds differently: at most one bf16 ulp, counted in the test),
- *       closed forms silu(0) = 0, silu(x) -> x and -> -0 for large |x|, h == b * silu(a) in double
+ *   oracle_swiglu_bf16                            pinned: torch's CPU F.silu and multiply on bf16 tensors, bit for
+ *       bit over every finite bf16 a; closed forms silu(0) = 0, silu(x) -> x and -> -0 for large |x|;
+ *       h == b * silu(a) in double within two bf16 roundings
+ *   oracle_swiglu_bwd_bf16                        pinned: torch's CPU autograd of the same two ops, bit for bit
+ *       over every finite bf16 a; float64 central differences; da(0) = dh b / 2, db = dh silu(a)
+ *   oracle_bias_gather_add / _bgrad               pinned: torch's inp + bias[ids] bit for bit, index_add_ in
+ *       float64, integer-valued data whose fp32 sums are exact in any order
  *   oracle_unpermute_combine                      pinned: brute force, torch restatement (index_copy_,
  *       multiply, sum) bit-exact for bf16 weights, inverse-of-permute property
  * Parity unpinned (nothing available here can pin it; the oracle's choice is stated instead):
