@@ -36,18 +36,13 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
-#ifndef AAMD_UNP_UNROLL
-#define AAMD_UNP_UNROLL 4
-#endif
-#ifndef AAMD_UNP_NT
-#define AAMD_UNP_NT 1
-#endif
-#pragma unroll AAMD_UNP_UNROLL
+    // four gathered rows in flight per lane; streaming loads: a permuted row is read exactly once
+#pragma unroll 4
     for (int j = 0; j < topk; j++) {
       const int r = srow[j];
       if (r < 0) continue;
       const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)r * H + c * 8);
-      const v4i raw = AAMD_UNP_NT ? __builtin_nontemporal_load(src) : *src;
+      const v4i raw = __builtin_nontemporal_load(src);
       float v[8];
       unpack8(raw, v);
       const float pv = sprob[j];

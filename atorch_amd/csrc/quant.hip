@@ -129,6 +129,8 @@ __device__ __forceinline__ v4i pack8_bf16(const float* v) {
 // 1x128 quant, 16 lanes per tile, U tiles per lane group.  SCATTER: write each quantised
 // row to its topk destinations (row_map), reading it once.
 // ---------------------------------------------------------------------------------------
+// tiles per 16-lane group and pass: two keep enough loads in flight (one and four measured slower)
+constexpr int kQuantU = 2;
 template <typename IN, bool SCATTER, int U>
 __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::elem* __restrict__ x, int64_t ldx,
                                                           int nt, int64_t total_tiles,
@@ -164,14 +166,8 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     if (!valid[u]) continue;
     if (h_out != nullptr)  // the gated activation itself, for callers that keep it
       *reinterpret_cast<v4i*>(h_out + row[u] * cols + (int64_t)tc[u] * kTile + l * 8) = pack8_bf16(v);
-#ifndef AAMD_QUANT_NT_STORE
-#define AAMD_QUANT_NT_STORE 1
-#endif
-    auto put = [&](v2i* dst, v2i val) {
-      // the codes are not read again by this kernel: streaming stores keep them out of the way
-      if (AAMD_QUANT_NT_STORE) __builtin_nontemporal_store(val, dst);
-      else *dst = val;
-    };
+    // the codes are not read again by this kernel: streaming stores keep them out of the way
+    auto put = [&](v2i* dst, v2i val) { __builtin_nontemporal_store(val, dst); };
     if constexpr (!SCATTER) {
       put(reinterpret_cast<v2i*>(q + row[u] * cols + (int64_t)tc[u] * kTile + l * 8), codes);
       if (l == 0) s[row[u] * nt + tc[u]] = sc;
@@ -504,10 +500,7 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   const int64_t total = T * nt;
   AAMD_REQUIRE(total < (int64_t)1 << 40, "quant_1x128: too many tiles");
   hipStream_t st = (hipStream_t)stream;
-#ifndef AAMD_QUANT_U
-#define AAMD_QUANT_U 2
-#endif
-  constexpr int U = AAMD_QUANT_U;
+  constexpr int U = kQuantU;
   const int64_t blocks = (total + 16 * U - 1) / (16 * U);
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "quant_1x128: grid too large");
   dim3 grid((unsigned)blocks), block(256);
@@ -573,7 +566,7 @@ extern "C" int aamd_swiglu_quant_1x128(const void* fc1, int64_t rows, int64_t F,
   const int nt = (int)(F / kTile);
   const int64_t total = rows * nt;
   AAMD_REQUIRE(total < (int64_t)1 << 40, "swiglu_quant: too many tiles");
-  constexpr int U = AAMD_QUANT_U;
+  constexpr int U = kQuantU;
   const int64_t blocks = (total + 16 * U - 1) / (16 * U);
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "swiglu_quant: grid too large");
   quant_1x128_kernel<GLU, false, U><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
