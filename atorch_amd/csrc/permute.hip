@@ -36,34 +36,54 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
-    // four gathered rows in flight per lane; streaming loads: a permuted row is read exactly once
-#pragma unroll 4
-    for (int j = 0; j < topk; j++) {
-      const int r = srow[j];
-      if (r < 0) continue;
-      const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)r * H + c * 8);
-      const v4i raw = __builtin_nontemporal_load(src);
-      float v[8];
-      unpack8(raw, v);
-      const float pv = sprob[j];
-      // separate multiply and add (no FMA contraction): the reference multiplies, rounds the
-      // product to the promoted dtype, then sums
+    // B gathered rows at a time: their loads are issued together, then folded in slot order.  (A
+    // plain loop over the slots compiles to one load in flight per lane.)  Streaming loads: a
+    // permuted row is read exactly once.
+    auto batch = [&](auto Bc, int j0) {
+      constexpr int B = decltype(Bc)::value;
+      v4i raw[B];
+      float pv[B];
 #pragma unroll
-      for (int i = 0; i < 8; i += 2) {
-        float p0 = v[i], p1 = v[i + 1];
-        if constexpr (PD == AAMD_BF16) {
-          const uint32_t pk = pack_bf16x2(v[i] * pv, v[i + 1] * pv);
-          p0 = __uint_as_float(pk << 16);
-          p1 = __uint_as_float(pk & 0xffff0000u);
-        }
-        if constexpr (PD == AAMD_F32) {
-          p0 = v[i] * pv;
-          p1 = v[i + 1] * pv;
-        }
-        acc[i] = acc[i] + p0;
-        acc[i + 1] = acc[i + 1] + p1;
+      for (int u = 0; u < B; u++) {
+        // row and weight are the same in every lane: held in scalar registers, the row address is
+        // scalar base + lane offset.  A dropped copy reads row 0 and is masked to the zeros the
+        // reference multiplies there.
+        const int r = __builtin_amdgcn_readfirstlane(srow[j0 + u]);
+        const int keep = r < 0 ? 0 : -1;
+        const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)(r < 0 ? 0 : r) * H) + c;
+        raw[u] = __builtin_nontemporal_load(src);
+#pragma unroll
+        for (int i = 0; i < 4; i++) raw[u][i] &= keep;
+        pv[u] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(sprob[j0 + u])));
       }
-    }
+#pragma unroll
+      for (int u = 0; u < B; u++) {
+        float v[8];
+        unpack8(raw[u], v);
+        // separate multiply and add (no FMA contraction): the reference multiplies, rounds the
+        // product to the promoted dtype, then sums
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+          float p0 = v[i], p1 = v[i + 1];
+          if constexpr (PD == AAMD_BF16) {
+            const uint32_t pk = pack_bf16x2(v[i] * pv[u], v[i + 1] * pv[u]);
+            p0 = __uint_as_float(pk << 16);
+            p1 = __uint_as_float(pk & 0xffff0000u);
+          }
+          if constexpr (PD == AAMD_F32) {
+            p0 = v[i] * pv[u];
+            p1 = v[i + 1] * pv[u];
+          }
+          acc[i] = acc[i] + p0;
+          acc[i + 1] = acc[i + 1] + p1;
+        }
+      }
+    };
+    int j = 0;
+    for (; j + 8 <= topk; j += 8) batch(std::integral_constant<int, 8>{}, j);
+    if (j + 4 <= topk) { batch(std::integral_constant<int, 4>{}, j); j += 4; }
+    if (j + 2 <= topk) { batch(std::integral_constant<int, 2>{}, j); j += 2; }
+    if (j < topk) batch(std::integral_constant<int, 1>{}, j);
     if constexpr (PD == AAMD_F32) {
       float* dst = reinterpret_cast<float*>(out) + t * H + c * 8;
       reinterpret_cast<v4f*>(dst)[0] = v4f{acc[0], acc[1], acc[2], acc[3]};
