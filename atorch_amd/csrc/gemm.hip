@@ -21,7 +21,8 @@
 // matrix pipe busy.
 //
 // Data path: global -> LDS directly (global_load_lds, 16 bytes per lane, no register stop),
-// two stages, one workgroup barrier per step.  Rows are 128 bytes; the 16-byte chunks of a row
+// two stages, one workgroup barrier per step (two in the 256x256 configuration, whose L tile is
+// requested two steps ahead).  Rows are 128 bytes; the 16-byte chunks of a row
 // are XOR-swizzled so that the linear 1 KB writes of the direct loads and the 32-row MFMA
 // operand reads are both bank-conflict free on the 64-bank LDS (measured: ~235 of 256 B/clk).
 #include <stdlib.h>
@@ -35,7 +36,6 @@ constexpr int kBK = 128;  // contraction bytes per step == scale block
 enum GemmMode { kRaggedRows = 0, kRaggedK = 1 };
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // XOR swizzle of the 16-byte chunk index inside a 128-byte LDS row (depends on row % 16 only).
