@@ -503,6 +503,57 @@ def test_grouped_gemm_wgrad(oracle, dev, M, N, K, E, mult):
             assert torch.equal(acc[e].cpu(), base[e])
 
 
+def test_tile_and_block_quant_match_torch_ops_on_the_gpu(dev):
+    """The reference formula (triton_kernel.py:21-46, 94-140: s = max(amax, eps) / 448, 0 -> 1,
+    code = e4m3fn(x / s)) written with torch ops and run on this GPU (tensor / tensor is an IEEE
+    division, the cast rounds to nearest even), against the kernels: bit for bit."""
+    from atorch_amd import kernels
+
+    g = torch.Generator().manual_seed(33)
+    x = (torch.randn(257, 1024, generator=g) * torch.exp(torch.randn(257, 1, generator=g) * 3)).bfloat16().to(dev)
+    x[5] = 0
+    t = x.float().view(257, 8, 128)
+    s_ref = t.abs().amax(dim=-1) / torch.full((), 448.0, device=dev)
+    s_ref = torch.where(s_ref == 0, torch.ones_like(s_ref), s_ref)
+    q_ref = (t / s_ref.unsqueeze(-1)).to(torch.float8_e4m3fn).view(257, 1024)
+    q, s = kernels.tile_quant(x)
+    assert torch.equal(s, s_ref) and torch.equal(_u8(q), _u8(q_ref))
+    w = (torch.randn(384, 512, generator=g) * 0.05).bfloat16().to(dev)
+    b = w.float().view(3, 128, 4, 128)
+    sb_ref = b.abs().amax(dim=(1, 3)) / torch.full((), 448.0, device=dev)
+    sb_ref = torch.where(sb_ref == 0, torch.ones_like(sb_ref), sb_ref)
+    qb_ref = (b / sb_ref[:, None, :, None]).to(torch.float8_e4m3fn).view(384, 512)
+    qb, sb = kernels.block_quant(w)
+    assert torch.equal(sb, sb_ref) and torch.equal(_u8(qb), _u8(qb_ref))
+
+
+def test_unpermute_matches_torch_ops_on_the_gpu(dev):
+    """The reference's own sequence (token_dispatcher.py:119-161: zeros, index_copy_, multiply by the
+    probabilities, sum over top-k) run with torch ops on this GPU, against the fused kernel: bit for bit
+    with bf16 probabilities (each product is rounded to bf16, the eight terms are summed in fp32 in slot
+    order and rounded once).  With fp32 probabilities torch's GPU reduction adds in another order, so
+    only closeness is asserted there."""
+    from atorch_amd import token_dispatcher
+
+    g = torch.Generator().manual_seed(31)
+    T, H, k, E = 1024, 512, 8, 16
+    x = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(dev)
+    sorted_idx = torch.argsort(ids.reshape(-1), stable=True)
+    y = x.index_select(0, sorted_idx // k)
+    for pd in (torch.bfloat16, torch.float32):
+        probs = torch.rand(T, k, generator=g).to(pd).to(dev)
+        un = torch.zeros(T * k, H, dtype=y.dtype, device=dev)
+        un.index_copy_(0, sorted_idx, y)
+        ref = (un.reshape(T, k, H) * probs.unsqueeze(-1)).sum(dim=1)
+        out = token_dispatcher.unpermute(y, sorted_idx, probs=probs)
+        assert out.dtype == ref.dtype
+        if pd == torch.bfloat16:
+            assert torch.equal(out, ref)
+        else:
+            assert float((out - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+
 # ------------------------------------------------------------------------------------------
 # f4: per-expert bias on expert-tagged rows
 # ------------------------------------------------------------------------------------------
