@@ -33,14 +33,18 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
   __syncthreads();
   const int64_t H = (int64_t)H8 * 8;
   for (int c = threadIdx.x; c < H8; c += blockDim.x) {
-    float acc[8];
+    // torch's reduction of a strided dimension, which the reference runs: four accumulators, slot j
+    // goes to accumulator j mod 4, the total is ((a0 + a1) + a2) + a3
+    float acc[4][8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[a][i] = 0.f;
     // B gathered rows at a time: their loads are issued together, then folded in slot order.  (A
     // plain loop over the slots compiles to one load in flight per lane.)  Streaming loads: a
     // permuted row is read exactly once.
-    auto batch = [&](auto Bc, int j0) {
-      constexpr int B = decltype(Bc)::value;
+    auto batch = [&](auto Bc, int j0, auto A0c) {
+      constexpr int B = decltype(Bc)::value, A0 = decltype(A0c)::value;  // A0 = j0 mod 4
       v4i raw[B];
       float pv[B];
 #pragma unroll
@@ -74,24 +78,33 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
             p0 = v[i] * pv[u];
             p1 = v[i + 1] * pv[u];
           }
-          acc[i] = acc[i] + p0;
-          acc[i + 1] = acc[i + 1] + p1;
+          acc[(A0 + u) & 3][i] = acc[(A0 + u) & 3][i] + p0;
+          acc[(A0 + u) & 3][i + 1] = acc[(A0 + u) & 3][i + 1] + p1;
         }
       }
     };
-    int j = 0;
-    for (; j + 8 <= topk; j += 8) batch(std::integral_constant<int, 8>{}, j);
-    if (j + 4 <= topk) { batch(std::integral_constant<int, 4>{}, j); j += 4; }
-    if (j + 2 <= topk) { batch(std::integral_constant<int, 2>{}, j); j += 2; }
-    if (j < topk) batch(std::integral_constant<int, 1>{}, j);
+    using std::integral_constant;
+    int j = 0;  // stays a multiple of 4 until the batch of two
+    for (; j + 8 <= topk; j += 8) batch(integral_constant<int, 8>{}, j, integral_constant<int, 0>{});
+    if (j + 4 <= topk) { batch(integral_constant<int, 4>{}, j, integral_constant<int, 0>{}); j += 4; }
+    if (j + 2 <= topk) {
+      batch(integral_constant<int, 2>{}, j, integral_constant<int, 0>{});
+      j += 2;
+      if (j < topk) batch(integral_constant<int, 1>{}, j, integral_constant<int, 2>{});
+    } else if (j < topk) {
+      batch(integral_constant<int, 1>{}, j, integral_constant<int, 0>{});
+    }
+    float tot[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) tot[i] = ((acc[0][i] + acc[1][i]) + acc[2][i]) + acc[3][i];
     if constexpr (PD == AAMD_F32) {
       float* dst = reinterpret_cast<float*>(out) + t * H + c * 8;
-      reinterpret_cast<v4f*>(dst)[0] = v4f{acc[0], acc[1], acc[2], acc[3]};
-      reinterpret_cast<v4f*>(dst)[1] = v4f{acc[4], acc[5], acc[6], acc[7]};
+      reinterpret_cast<v4f*>(dst)[0] = v4f{tot[0], tot[1], tot[2], tot[3]};
+      reinterpret_cast<v4f*>(dst)[1] = v4f{tot[4], tot[5], tot[6], tot[7]};
     } else {
       v4i w;
 #pragma unroll
-      for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
+      for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(tot[2 * i], tot[2 * i + 1]);
       *reinterpret_cast<v4i*>(reinterpret_cast<u16*>(out) + t * H + c * 8) = w;
     }
   }

@@ -185,7 +185,8 @@ int aamd_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uin
  *   out[t, :] = sum_j probs[t, j] * y[row_map[t*topk + j], :]
  * Replaces unpermute, token_dispatcher.py:119-161 (zeros + index_copy_ + multiply + sum).
  * Each product is rounded to the promoted dtype before the fp32 sum, as the reference's
- * separate multiply and sum do (:156-159).
+ * separate multiply and sum do (:156-159); the sum adds in the order of torch's GPU reduction
+ * (slot j into accumulator j mod 4, then ((a0 + a1) + a2) + a3).
  *   y [M, H] bf16; row_map [T*topk] int32 (-1 = dropped copy, contributes 0)
  *   probs [T, topk] of probs_dtype (AAMD_BF16 -> out bf16; AAMD_F32 -> out fp32;
  *   AAMD_NONE -> probs ignored, out bf16); H % 8 == 0.

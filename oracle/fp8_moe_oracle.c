@@ -34,14 +34,13 @@
  *   oracle_bias_gather_add / _bgrad               pinned: torch's inp + bias[ids] bit for bit, index_add_ in
  *       float64, integer-valued data whose fp32 sums are exact in any order
  *   oracle_unpermute_combine                      pinned: brute force, torch restatement (index_copy_,
- *       multiply, sum) bit-exact for bf16 weights, inverse-of-permute property
+ *       multiply, sum) bit-exact for bf16 weights, inverse-of-permute property; the summation order
+ *       (four interleaved accumulators) is pinned against torch's own sum on the GPU by a GPU test
  * Parity unpinned (nothing available here can pin it; the oracle's choice is stated instead):
  *   - the exact fp32 rounding of the reference's compiled Triton division x / s on its GPU: the oracle
  *     is defined as IEEE round-to-nearest division;
  *   - the numerics and layouts of the external `kitchen` package behind quantize_op (not in the
- *     reference tree, no version pinned): the in-tree Triton formulas are the anchor instead;
- *   - the summation order of torch's GPU `sum(dim=1)` in unpermute for fp32 weights: the oracle sums the
- *     top-k terms sequentially in fp32.
+ *     reference tree, no version pinned): the in-tree Triton formulas are the anchor instead.
  *
  * Build: gcc -O2 -fno-fast-math -ffp-contract=off -shared -fPIC (see Makefile).
  */
@@ -299,9 +298,10 @@ int oracle_permute_indices(const int64_t *ids, int64_t n, int64_t E, int64_t *so
  *       accumulate, one final rounding
  * probs_is_bf16: probs bf16 -> products and result bf16 (out_bf16 written);
  * else probs fp32 -> products and result fp32 (out_f32 written).
- * The fp32 accumulation is sequential over slot 0..k-1; torch's own reduce
- * order is an implementation detail, so bit parity with torch is not claimed
- * for k > 2 (difference <= 1 ulp of the output type).
+ * The fp32 accumulation follows torch's GPU reduction of a strided dimension, which is what the
+ * reference executes: four accumulators, slot j goes to accumulator j mod 4 in slot order, then
+ * ((a0 + a1) + a2) + a3.  (For k <= 4 that is the plain left-to-right sum.)  A GPU test checks this
+ * order against torch's own sum on the device.
  * probs == NULL: topk = 1, plain inverse permutation (:141-144).
  * n_perm may be smaller than T*k (rows dropped): missing rows count as 0.
  */
@@ -321,7 +321,7 @@ int oracle_unpermute_combine(const uint16_t *y, int64_t n_perm, int64_t H, const
     }
     for (int64_t t = 0; t < T; t++)
         for (int64_t h = 0; h < H; h++) {
-            float acc = 0.0f;
+            float acc4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             for (int64_t j = 0; j < k; j++) {
                 int64_t row = inv[t * k + j];
                 float v = row < 0 ? 0.0f : bf16_to_f32(y[row * H + h]);
@@ -333,8 +333,9 @@ int oracle_unpermute_combine(const uint16_t *y, int64_t n_perm, int64_t H, const
                         v = v * ((const float *)probs)[t * k + j];
                     }
                 }
-                acc += v;
+                acc4[j & 3] += v;
             }
+            const float acc = ((acc4[0] + acc4[1]) + acc4[2]) + acc4[3];
             if (probs && !probs_is_bf16)
                 out_f32[t * H + h] = acc;
             else
