@@ -131,6 +131,30 @@ def test_swiglu_bwd_quant_dual_grouped(oracle, dev, M, F, E):
     assert torch.equal(_u8(q_t3[:, :ptot]), _u8(q_t[:, :ptot])) and torch.equal(s_t3[: ptot // TILE], s_t[: ptot // TILE])
 
 
+def test_swiglu_forward_and_backward_against_torch_on_the_gpu(dev):
+    """The reference's two torch ops and their autograd, run on this GPU, against the fused kernels:
+    the same bounds as against the oracle (one bf16 ulp where sigmoid enters once, two where a bf16
+    product with it is rounded again), on a small fraction of elements."""
+    from atorch_amd import kernels
+
+    g = torch.Generator().manual_seed(41)
+    M, F = 640, 512
+    fc1 = (torch.randn(M, 2 * F, generator=g) * 2).bfloat16().to(dev)
+    dh = torch.randn(M, F, generator=g).bfloat16().to(dev)
+    leaf = fc1.clone().requires_grad_(True)
+    a, b = torch.chunk(leaf, 2, dim=-1)
+    h_ref = torch.nn.functional.silu(a) * b
+    h_ref.backward(dh)
+    _, _, h = kernels.swiglu_tile_quant(fc1, return_activation=True)
+    goff = kernels.group_offsets_from_splits([M], dev)
+    _, _, _, _, gr = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, 1, return_grad=True)
+    for got, ref in ((h, h_ref.detach()), (gr, leaf.grad)):
+        d = _ulp_diff(got.cpu(), ref.cpu())
+        d = torch.where(got.cpu().float() == ref.cpu().float(), torch.zeros_like(d), d)
+        assert int(d.max()) <= 2, int(d.max())
+        assert float((d > 0).float().mean()) < 2e-3
+
+
 def test_swiglu_quant_rejects_bad_shapes(dev):
     from atorch_amd import kernels
 
