@@ -574,10 +574,26 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     // Loads complete in issue order, so "all but the newest L group" is one wait count.  Past the
     // end the loads re-read the last block to keep the counts uniform.
     auto kclamp = [&](int k) { return k < nkb ? k : nkb - 1; };
+#ifdef AAMD_GEMM_BARSTAT
+    // measurement build: cycles this wave spends waiting for its loads, in the end-of-step barrier
+    // and in the mid-step barrier
+    unsigned long long bs_load = 0, bs_end = 0, bs_mid = 0;
+    auto wait_all_but_newest_l = [&]() {
+      const unsigned long long t0 = __builtin_readcyclecounter();
+      if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(C::LCH + kScaleLd) : "memory");
+      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(C::LCH) : "memory");
+      const unsigned long long t1 = __builtin_readcyclecounter();
+      asm volatile("s_barrier" ::: "memory");
+      const unsigned long long t2 = __builtin_readcyclecounter();
+      bs_load += t1 - t0;
+      bs_end += t2 - t1;
+    };
+#else
     auto wait_all_but_newest_l = [&]() {
       if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
       else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
     };
+#endif
     if (nkb > 0) {
       dmaL(0, Lbuf0, Sc0);
       dmaR(0, Rbuf0, Sc0);
@@ -595,7 +611,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
         static_assert(C::RCH % RT == 0 && RT + C::LCH <= NTILES, "spread schedule");
         const int kr = kclamp(kb + 1), kl = kclamp(kb + 2);
         auto mid = [&]() {
+#ifdef AAMD_GEMM_BARSTAT
+          const unsigned long long t0 = __builtin_readcyclecounter();
+#endif
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
+#ifdef AAMD_GEMM_BARSTAT
+          bs_mid += __builtin_readcyclecounter() - t0;
+#endif
           if (kLoads && !kMath) dmaL(kl, Lc, Sc);
           else if (kLoads) dmaL_scales(kl, Sc);
         };
@@ -622,6 +644,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       }
       if (kb < nkb) step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
+#ifdef AAMD_GEMM_BARSTAT
+      if (wave == (int)(blockIdx.x & 7) && lane == 0 && p.bias != nullptr) {
+        unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 8;
+        dst[0] = bs_load; dst[1] = bs_end; dst[2] = bs_mid; dst[3] = __builtin_readcyclecounter() - stamp[3];
+        dst[4] = wave; dst[5] = nkb;
+      }
+#endif
     }
   }
 
@@ -719,10 +748,12 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   stamp[5] = __builtin_readcyclecounter();
   stamp[2] = __builtin_amdgcn_s_memrealtime();  // constant-rate clock at the end (overwrites the loads-issued stamp)
+#ifndef AAMD_GEMM_BARSTAT
   if (tid == 0 && p.bias != nullptr) {
     unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 8;
     for (int i = 0; i < 8; i++) dst[i] = stamp[i];
   }
+#endif
 #endif
 }
 
