@@ -151,7 +151,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   constexpr int kLsBatch = MODE == kRaggedRows ? BM * 8 * 4 : 0;
   static_assert(NT == 2 * BM, "two threads fetch the 32 bytes of a row's scale batch");
   __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4 + 2 * kLsBatch];
-  __shared__ int slot;
+  struct Lookup { int64_t l0; int total, g, lvalid; };
+  __shared__ Lookup look;
   // both L stages first, then both R stages: every fragment of a side is within 64 KB of one base
   // address, so the stage and the sub-tile row go into the immediate offset of the LDS reads
   uint8_t* const Lbuf0 = lds;
@@ -182,8 +183,29 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // hardware's own dispatch balances ragged tiles better).  Workgroup ids go round-robin over
   // the 8 XCDs; every XCD gets one contiguous range of tile ids so that tiles sharing operand
   // panels meet in the same L2.
-  const int total_lt = MODE == kRaggedRows ? (p.goff ? p.tile_off[p.E] : (int)((p.Lrows + BM - 1) / BM))
-                                           : p.nLt * p.E;
+  // Row-ragged launches look their group up in the device-side offsets.  Every load of that lookup
+  // goes out before the first wait: thread e fetches the tile range and the row range of group e,
+  // thread 0 the tile count besides, so the lookup costs one trip to memory instead of three
+  // dependent ones (tile count -> tile index -> matching group -> its row offsets).
+  int total_lt;
+  int t_lo = 0, t_hi = 0;
+  int64_t r_lo = 0, r_hi = 0;
+  if (MODE == kRaggedRows && p.goff != nullptr) {
+    if (tid < p.E) {
+      t_lo = p.tile_off[tid];
+      t_hi = p.tile_off[tid + 1];
+      r_lo = p.goff[tid];
+      r_hi = p.goff[tid + 1];
+    }
+    if (tid == 0) {
+      look.total = p.tile_off[p.E];
+      look.g = p.E + 1;
+    }
+    __syncthreads();
+    total_lt = look.total;
+  } else {
+    total_lt = MODE == kRaggedRows ? (int)((p.Lrows + BM - 1) / BM) : p.nLt * p.E;
+  }
   const int64_t ntot = (int64_t)total_lt * p.nRt;
   const int64_t bid = blockIdx.x;
   if (bid >= ntot) return;
@@ -210,11 +232,22 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   int kb0, nkb;   // contraction blocks [kb0, kb0 + nkb)
   if constexpr (MODE == kRaggedRows) {
     if (p.goff) {
-      g = find_group(p.tile_off, p.E, lt, &slot);
+      // exactly one group holds tile lt (empty groups hold none)
+      auto claim = [&](int e, int lo, int hi, int64_t rows_lo, int64_t rows_hi) {
+        if (lt >= lo && lt < hi) {
+          const int64_t first = rows_lo + (int64_t)(lt - lo) * BM, left = rows_hi - first;
+          look.g = e;
+          look.l0 = first;
+          look.lvalid = left < BM ? (int)left : BM;
+        }
+      };
+      if (tid < p.E) claim(tid, t_lo, t_hi, r_lo, r_hi);
+      for (int e = tid + NT; e < p.E; e += NT) claim(e, p.tile_off[e], p.tile_off[e + 1], p.goff[e], p.goff[e + 1]);
+      __syncthreads();
+      g = look.g;
       if (g >= p.E) return;
-      l0 = p.goff[g] + (int64_t)(lt - p.tile_off[g]) * BM;
-      const int64_t left = p.goff[g + 1] - l0;
-      lvalid = left < BM ? (int)left : BM;
+      l0 = look.l0;
+      lvalid = look.lvalid;
     } else {
       g = 0;
       l0 = (int64_t)lt * BM;
@@ -744,10 +777,14 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     else flush(u16{});
   }
 #ifdef AAMD_GEMM_TIMING
+#ifndef AAMD_GEMM_TIMING_PROLOGUE  // that build keeps the group-lookup and loads-issued stamps instead
   stamp[1] = __builtin_readcyclecounter();  // epilogue issued (overwrites the group-lookup stamp)
+#endif
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   stamp[5] = __builtin_readcyclecounter();
+#ifndef AAMD_GEMM_TIMING_PROLOGUE
   stamp[2] = __builtin_amdgcn_s_memrealtime();  // constant-rate clock at the end (overwrites the loads-issued stamp)
+#endif
 #ifndef AAMD_GEMM_BARSTAT
   if (tid == 0 && p.bias != nullptr) {
     unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 8;
