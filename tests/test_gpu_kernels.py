@@ -622,3 +622,33 @@ def test_bias_gather_add_autograd_and_edges(oracle, dev):
         bias_gather_add_fw(torch.zeros(4, 12, dtype=torch.bfloat16, device=dev), torch.zeros(2, 12, dtype=torch.bfloat16, device=dev),
                            torch.zeros(4, dtype=torch.int64, device=dev))  # 24-byte rows
 
+
+
+@pytest.mark.parametrize("M,N,K,E", [(4096, 128, 128, 700), (140000, 512, 128, 700)], ids=["tiles128", "tiles256"])
+def test_grouped_gemm_more_groups_than_threads(oracle, dev, M, N, K, E):
+    """More groups than a workgroup has threads (256 and 512 in the two tile configurations), most
+    of them tiny and many empty: the group lookup of a tile then needs more than one pass over the
+    offsets.  Reference: dequantise and multiply in float64, expert by expert."""
+    from atorch_amd import kernels
+
+    g = torch.Generator().manual_seed(E + M)
+    x = randn_bf16((M, K), 3)
+    w = randn_bf16((E, N, K), 4, std=0.02)
+    cuts = torch.sort(torch.randint(0, M + 1, (E - 1,), generator=g)).values
+    cuts[100:300] = cuts[100]  # a run of empty groups
+    cuts = torch.sort(cuts).values.tolist()
+    b = [0] + cuts + [M]
+    splits = [b[i + 1] - b[i] for i in range(E)]
+    assert sum(splits) == M and splits.count(0) >= 199
+    qx, sx = kernels.tile_quant(x.to(dev))
+    qw, sw, _, _ = kernels.block_quant_batched(w.to(dev))
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    y = kernels.grouped_gemm_nt(qx, sx, qw, sw, goff, out_dtype=torch.float32).cpu()
+    xd = oracle.torch_dequant_tile(qx.cpu().view(torch.uint8), sx.cpu()).double()
+    ref = torch.zeros(M, N, dtype=torch.float64)
+    off = 0
+    for e, m in enumerate(splits):
+        if m:
+            ref[off : off + m] = xd[off : off + m] @ oracle.torch_dequant_block(qw[e].cpu().view(torch.uint8), sw[e].cpu()).double().t()
+        off += m
+    assert rel_err(y, ref.float()) <= GEMM_TOL_F32
