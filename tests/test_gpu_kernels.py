@@ -377,7 +377,7 @@ def test_block_quant_matches_oracle(oracle, dev, dtype, E, N, K):
 # a3: row-wise + transposed quant of ragged groups
 # ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M,K,E,mult", [(512, 256, 4, 128), (1000, 384, 6, 16), (777, 128, 5, 1)])
+@pytest.mark.parametrize("M,K,E,mult", [(512, 256, 4, 128), (1000, 384, 6, 16), (777, 128, 5, 1), (3000, 128, 700, 1)])
 def test_dual_grouped_quant(oracle, dev, dtype, M, K, E, mult):
     from atorch_amd import kernels
 
@@ -497,7 +497,7 @@ def test_grouped_gemm_nt(oracle, dev, M, N, K, E, mult):
         off += m
 
 
-@pytest.mark.parametrize("M,N,K,E,mult", [(512, 128, 256, 4, 128), (1000, 256, 128, 6, 16), (333, 128, 128, 3, 1)])
+@pytest.mark.parametrize("M,N,K,E,mult", [(512, 128, 256, 4, 128), (1000, 256, 128, 6, 16), (333, 128, 128, 3, 1), (3000, 128, 128, 700, 1)])
 def test_grouped_gemm_wgrad(oracle, dev, M, N, K, E, mult):
     from atorch_amd import kernels
 
