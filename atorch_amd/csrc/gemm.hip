@@ -64,6 +64,7 @@ struct GemmParams {
   int nLt;         // kRaggedK: L tiles
   int max_kb;      // kRaggedK: contraction blocks the operand buffers hold (ld_t / 128)
   int accumulate;
+  int group_r;     // kRaggedK: the tile order groups R tiles instead of L tiles
   int bias_dtype;
   int gl;          // L tiles that share an R panel in the tile order
   int ls_batch;    // kRaggedRows: L scales are fetched eight contraction blocks at a time
@@ -216,12 +217,25 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     const int64_t pid = xcd < rem ? xcd * (per + 1) + idx : rem * (per + 1) + (xcd - rem) * per + idx;
     // inside the range: groups of GL L tiles, R tile index outer, L tile inner
     const int GL = p.gl;
-    const int64_t width = (int64_t)GL * p.nRt;
-    const int first = (int)(pid / width) * GL;
-    const int gsz = total_lt - first < GL ? total_lt - first : GL;
-    const int in_grp = (int)(pid % width);
-    lt = first + in_grp % gsz;
-    rt = in_grp / gsz;
+    if (MODE == kRaggedK && p.group_r) {
+      // wgrad with more R tiles than L tiles: groups of GL R tiles, all L tiles of the expert inside
+      const int64_t per_e = (int64_t)p.nLt * p.nRt;
+      const int e = (int)(pid / per_e);
+      const int64_t pe = pid - e * per_e;
+      const int64_t width = (int64_t)GL * p.nLt;
+      const int first = (int)(pe / width) * GL;
+      const int gsz = p.nRt - first < GL ? p.nRt - first : GL;
+      const int in_grp = (int)(pe % width);
+      rt = first + in_grp % gsz;
+      lt = e * p.nLt + in_grp / gsz;
+    } else {
+      const int64_t width = (int64_t)GL * p.nRt;
+      const int first = (int)(pid / width) * GL;
+      const int gsz = total_lt - first < GL ? total_lt - first : GL;
+      const int in_grp = (int)(pid % width);
+      lt = first + in_grp % gsz;
+      rt = in_grp / gsz;
+    }
 #if defined(AAMD_GEMM_ABLATE) && (AAMD_GEMM_ABLATE == 3 || AAMD_GEMM_HOT == 1)
     lt = 0; rt = 0;  // measurement build: every workgroup streams the same tile
 #endif
@@ -834,6 +848,8 @@ static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st
   // at 4096 tokens per expert and 28672 x 4096 outputs, within 3 % either way elsewhere)
   p.gl = MODE == kRaggedK ? 4 : 8;
   if (const char* env = getenv("AAMD_GEMM_GL")) p.gl = atoi(env) > 0 ? atoi(env) : p.gl;
+  p.group_r = MODE == kRaggedK && p.nRt > p.nLt;
+  if (const char* env = getenv("AAMD_GEMM_GROUP_R")) p.group_r = atoi(env) != 0;
 
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "grouped_gemm: grid too large");
   dim3 grid((unsigned)blocks), block(C::NT);
