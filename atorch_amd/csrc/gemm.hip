@@ -64,7 +64,7 @@ struct GemmParams {
   int nLt;         // kRaggedK: L tiles
   int max_kb;      // kRaggedK: contraction blocks the operand buffers hold (ld_t / 128)
   int accumulate;
-  int group_r;     // kRaggedK: the tile order groups R tiles instead of L tiles
+  int group_r;     // the tile order groups R tiles (inside each group of rows / expert) instead of L tiles
   int bias_dtype;
   int gl;          // L tiles that share an R panel in the tile order
   int ls_batch;    // kRaggedRows: L scales are fetched eight contraction blocks at a time
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   constexpr int kLsBatch = MODE == kRaggedRows ? BM * 8 * 4 : 0;
   static_assert(NT == 2 * BM, "two threads fetch the 32 bytes of a row's scale batch");
   __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4 + 2 * kLsBatch];
-  struct Lookup { int64_t l0; int total, g, lvalid; };
+  struct Lookup { int64_t l0; int total, g, lvalid, rt; };
   __shared__ Lookup look;
   // both L stages first, then both R stages: every fragment of a side is within 64 KB of one base
   // address, so the stage and the sub-tile row go into the immediate offset of the LDS reads
@@ -211,12 +211,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   const int64_t bid = blockIdx.x;
   if (bid >= ntot) return;
   int g, lt, rt;
+  const int64_t per = ntot / 8, rem = ntot % 8;
+  const int64_t xcd = bid % 8, idx = bid / 8;
+  const int64_t pid = xcd < rem ? xcd * (per + 1) + idx : rem * (per + 1) + (xcd - rem) * per + idx;
+  const int GL = p.gl;
+  const bool by_group = MODE == kRaggedRows && p.goff != nullptr && p.group_r;  // tile order per group, below
   {
-    const int64_t per = ntot / 8, rem = ntot % 8;
-    const int64_t xcd = bid % 8, idx = bid / 8;
-    const int64_t pid = xcd < rem ? xcd * (per + 1) + idx : rem * (per + 1) + (xcd - rem) * per + idx;
     // inside the range: groups of GL L tiles, R tile index outer, L tile inner
-    const int GL = p.gl;
     if (MODE == kRaggedK && p.group_r) {
       // wgrad with more R tiles than L tiles: groups of GL R tiles, all L tiles of the expert inside
       const int64_t per_e = (int64_t)p.nLt * p.nRt;
@@ -247,9 +248,27 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   if constexpr (MODE == kRaggedRows) {
     if (p.goff) {
       // exactly one group holds tile lt (empty groups hold none)
+      // With group_r the tile ids of a group are contiguous and ordered in batches of GL R tiles,
+      // all L tiles of the group inside a batch, R index fastest: the weights of the group, the
+      // large operand, are then fetched once, and the group's few L panels are what gets re-read.
       auto claim = [&](int e, int lo, int hi, int64_t rows_lo, int64_t rows_hi) {
-        if (lt >= lo && lt < hi) {
-          const int64_t first = rows_lo + (int64_t)(lt - lo) * BM, left = rows_hi - first;
+        int my_lt = lt;
+        bool mine = lt >= lo && lt < hi;
+        if (by_group) {
+          const int64_t p_lo = (int64_t)lo * p.nRt, p_hi = (int64_t)hi * p.nRt;
+          mine = pid >= p_lo && pid < p_hi;
+          if (mine) {
+            const int nl = hi - lo;
+            const int64_t pe = pid - p_lo, width = (int64_t)GL * nl;
+            const int first_r = (int)(pe / width) * GL;
+            const int gsz = p.nRt - first_r < GL ? p.nRt - first_r : GL;
+            const int in_grp = (int)(pe % width);
+            look.rt = first_r + in_grp % gsz;
+            my_lt = lo + in_grp / gsz;
+          }
+        }
+        if (mine) {
+          const int64_t first = rows_lo + (int64_t)(my_lt - lo) * BM, left = rows_hi - first;
           look.g = e;
           look.l0 = first;
           look.lvalid = left < BM ? (int)left : BM;
@@ -262,6 +281,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       if (g >= p.E) return;
       l0 = look.l0;
       lvalid = look.lvalid;
+      if (by_group) rt = look.rt;
     } else {
       g = 0;
       l0 = (int64_t)lt * BM;
@@ -847,9 +867,14 @@ static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st
   // panels run over all tokens of an expert and are several times larger (measured: 5 % faster
   // at 4096 tokens per expert and 28672 x 4096 outputs, within 3 % either way elsewhere)
   p.gl = MODE == kRaggedK ? 4 : 8;
+  // group along the side with more tiles per expert (row-ragged launches: batches of 4 R tiles measured 1 % faster
+  // than the L grouping with many small groups, the same with few large ones)
+  if (MODE == kRaggedK) p.group_r = p.nRt > p.nLt;
+  else p.group_r = p.goff != nullptr && (int64_t)p.nRt * C::BM * p.E > p.Lrows;
+  if (MODE == kRaggedRows && p.group_r) p.gl = 4;
+  // overrides for experiments and tests
+  if (const char* env = getenv("AAMD_GEMM_GROUP_R")) p.group_r = atoi(env) != 0 && (MODE == kRaggedK || p.goff != nullptr);
   if (const char* env = getenv("AAMD_GEMM_GL")) p.gl = atoi(env) > 0 ? atoi(env) : p.gl;
-  p.group_r = MODE == kRaggedK && p.nRt > p.nLt;
-  if (const char* env = getenv("AAMD_GEMM_GROUP_R")) p.group_r = atoi(env) != 0;
 
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "grouped_gemm: grid too large");
   dim3 grid((unsigned)blocks), block(C::NT);
