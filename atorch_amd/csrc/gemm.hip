@@ -763,8 +763,11 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   uint8_t* const stg = lds + wave * kStgBytes;
   constexpr int WROWS = C::WTL * 32;
   static_assert(WROWS <= 64 && WROWS % 8 == 0, "the staging region holds 64 rows");
-  auto flush = [&](auto tag) {
+  // (the bias is a compile-time case: without one the staging is two conversions and a write per
+  // four values instead of a uniform branch, four adds and the moves that feed them)
+  auto flush = [&](auto tag, auto with_bias) {
     using ST = decltype(tag);  // staging type: OUT, or float when the old output is added in fp32
+    constexpr bool kBias = decltype(with_bias)::value;
     constexpr int CW = 128 / (int)sizeof(ST);  // columns per chunk
     constexpr int SUBS = CW / 32;              // 32-column sub-tiles per chunk
     constexpr int PITCH = 128 + (sizeof(ST) == 2 ? 8 : 16);
@@ -779,11 +782,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
         for (int q = 0; q < 4; q++) {
           const int64_t rcol = r0 + wrow0 + i * 32 + 8 * q + 4 * hg;
           v4f b4 = {0.f, 0.f, 0.f, 0.f};
-#ifdef AAMD_GEMM_TIMING
-          if (false) {
-#else
-          if (MODE == kRaggedRows && p.bias != nullptr) {
-#endif
+          if constexpr (kBias) {
             if (p.bias_dtype == AAMD_F32) {
               b4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(p.bias) + g * p.bias_group_stride + rcol);
             } else {
@@ -796,7 +795,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
           }
 #pragma unroll
           for (int j = 0; j < C::WTL; j++) {
-            const v4f o = v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]} + b4;
+            v4f o = v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            if constexpr (kBias) o += b4;
             uint8_t* dst = stg + (j * 32 + l32) * PITCH + (si * 32 + 8 * q + 4 * hg) * (int)sizeof(ST);
             if constexpr (sizeof(ST) == 4) {
               *reinterpret_cast<v4f*>(dst) = o;
@@ -850,11 +850,24 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       __builtin_amdgcn_wave_barrier();  // the next chunk overwrites the region
     }
   };
+#ifdef AAMD_GEMM_TIMING
+  const bool with_bias = false;  // the bias pointer carries the time stamps in that build
+#else
+  const bool with_bias = MODE == kRaggedRows && p.bias != nullptr;
+#endif
+  auto flush_as = [&](auto tag) {
+    if constexpr (MODE == kRaggedRows) {
+      if (with_bias) flush(tag, std::true_type{});
+      else flush(tag, std::false_type{});
+    } else {
+      flush(tag, std::false_type{});
+    }
+  };
   if constexpr (sizeof(OUT) == 4) {
-    flush(float{});
+    flush_as(float{});
   } else {
-    if (p.accumulate) flush(float{});
-    else flush(u16{});
+    if (p.accumulate) flush_as(float{});
+    else flush_as(u16{});
   }
 #ifdef AAMD_GEMM_TIMING
 #ifndef AAMD_GEMM_TIMING_PROLOGUE  // that build keeps the group-lookup and loads-issued stamps instead
