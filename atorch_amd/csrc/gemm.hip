@@ -820,8 +820,26 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
         raws[ps] = *reinterpret_cast<const v4i*>(stg + (ps * 8 + (lane >> 3)) * PITCH + (lane & 7) * 16);
 #pragma unroll
       for (int ps = 0; ps < WROWS / 8; ps++) asm volatile("" : "+v"(raws[ps]));
-      OUT* out_row = Cg + (l0 + wlrow0 + (lane >> 3)) * p.ldc + col;
+      OUT* const out_row0 = Cg + (l0 + wlrow0 + (lane >> 3)) * p.ldc + col;
       const int64_t row_step = 8 * p.ldc;
+      // accumulation into an fp32 output: the old values of all rows are requested before the
+      // first is used (one trip to memory per chunk instead of one per row)
+      constexpr bool kAddF32 = sizeof(ST) == sizeof(OUT) && sizeof(OUT) == 4;
+      v4f olds[kAddF32 ? WROWS / 8 : 1];
+      if constexpr (kAddF32) {
+        if (p.accumulate) {
+          OUT* o_row = out_row0;
+#pragma unroll
+          for (int ps = 0; ps < WROWS / 8; ps++) {
+            olds[ps] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (wlrow0 + ps * 8 + (lane >> 3) < lvalid) olds[ps] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(o_row));
+            o_row += row_step;
+          }
+#pragma unroll
+          for (int ps = 0; ps < WROWS / 8; ps++) asm volatile("" : "+v"(olds[ps]));
+        }
+      }
+      OUT* out_row = out_row0;
 #pragma unroll
       for (int ps = 0; ps < WROWS / 8; ps++) {
         const int lrow = wlrow0 + ps * 8 + (lane >> 3);
@@ -834,8 +852,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
               // the output is not read again by this launch: streaming stores keep it from
               // evicting operand panels from L2 (measured +1-2 % where the output is large)
               if (p.accumulate) {
-                const v4f o = __builtin_bit_cast(v4f, raw) + *reinterpret_cast<const v4f*>(out);
-                *reinterpret_cast<v4f*>(out) = o;
+                const v4f o = __builtin_bit_cast(v4f, raw) + olds[ps];
+                __builtin_nontemporal_store(o, reinterpret_cast<v4f*>(out));
               } else {
                 __builtin_nontemporal_store(raw, reinterpret_cast<v4i*>(out));
               }
