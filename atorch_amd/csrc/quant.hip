@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     const v2i codes = quant8(v, sc, plain_div);
     if (!valid[u]) continue;
     if (h_out != nullptr)  // the gated activation itself, for callers that keep it
-      *reinterpret_cast<v4i*>(h_out + row[u] * cols + (int64_t)tc[u] * kTile + l * 8) = pack8_bf16(v);
+      __builtin_nontemporal_store(pack8_bf16(v), reinterpret_cast<v4i*>(h_out + row[u] * cols + (int64_t)tc[u] * kTile + l * 8));
     // the codes are not read again by this kernel: streaming stores keep them out of the way
     auto put = [&](v2i* dst, v2i val) { __builtin_nontemporal_store(val, dst); };
     if constexpr (!SCATTER) {
@@ -303,7 +303,7 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
 #pragma unroll
     for (int j = 0; j < 8; j++) cm[j] = fmaxf(cm[j], fabsf(v[i][j]));
     if (h_out != nullptr && gr * 8 + i < mvalid)
-      *reinterpret_cast<v4i*>(h_out + (m0 + gr * 8 + i) * cols + (int64_t)kc * kTile + c * 8) = pack8_bf16(v[i]);
+      __builtin_nontemporal_store(pack8_bf16(v[i]), reinterpret_cast<v4i*>(h_out + (m0 + gr * 8 + i) * cols + (int64_t)kc * kTile + c * 8));
     if (q != nullptr) {
       const float sc = scale_from_amax(row16_max(amax8(v[i])), eps);
       const int r = gr * 8 + i;
