@@ -152,8 +152,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   constexpr int kLsBatch = MODE == kRaggedRows ? BM * 8 * 4 : 0;
   static_assert(NT == 2 * BM, "two threads fetch the 32 bytes of a row's scale batch");
   __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStage + 2 * NT * 4 + 2 * kLsBatch];
-  struct Lookup { int64_t l0; int total, g, lvalid, rt; };
-  __shared__ Lookup look;
   // both L stages first, then both R stages: every fragment of a side is within 64 KB of one base
   // address, so the stage and the sub-tile row go into the immediate offset of the LDS reads
   uint8_t* const Lbuf0 = lds;
@@ -184,26 +182,22 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // hardware's own dispatch balances ragged tiles better).  Workgroup ids go round-robin over
   // the 8 XCDs; every XCD gets one contiguous range of tile ids so that tiles sharing operand
   // panels meet in the same L2.
-  // Row-ragged launches look their group up in the device-side offsets.  Every load of that lookup
-  // goes out before the first wait: thread e fetches the tile range and the row range of group e,
-  // thread 0 the tile count besides, so the lookup costs one trip to memory instead of three
-  // dependent ones (tile count -> tile index -> matching group -> its row offsets).
+  // Row-ragged launches look their group up in the device-side offsets.  Every wave does it on its
+  // own, without LDS or barriers: lane e fetches the tile range and the row range of group e (all
+  // loads go out before the first wait: one trip to memory instead of three dependent ones, tile
+  // count -> tile index -> matching group -> its row offsets), the lane whose group holds the tile
+  // is found with a ballot and its values are broadcast with readlane.
   int total_lt;
   int t_lo = 0, t_hi = 0;
   int64_t r_lo = 0, r_hi = 0;
   if (MODE == kRaggedRows && p.goff != nullptr) {
-    if (tid < p.E) {
-      t_lo = p.tile_off[tid];
-      t_hi = p.tile_off[tid + 1];
-      r_lo = p.goff[tid];
-      r_hi = p.goff[tid + 1];
+    if (lane < p.E) {
+      t_lo = p.tile_off[lane];
+      t_hi = p.tile_off[lane + 1];
+      r_lo = p.goff[lane];
+      r_hi = p.goff[lane + 1];
     }
-    if (tid == 0) {
-      look.total = p.tile_off[p.E];
-      look.g = p.E + 1;
-    }
-    __syncthreads();
-    total_lt = look.total;
+    total_lt = p.tile_off[p.E];
   } else {
     total_lt = MODE == kRaggedRows ? (int)((p.Lrows + BM - 1) / BM) : p.nLt * p.E;
   }
@@ -251,37 +245,47 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       // With group_r the tile ids of a group are contiguous and ordered in batches of GL R tiles,
       // all L tiles of the group inside a batch, R index fastest: the weights of the group, the
       // large operand, are then fetched once, and the group's few L panels are what gets re-read.
-      auto claim = [&](int e, int lo, int hi, int64_t rows_lo, int64_t rows_hi) {
-        int my_lt = lt;
-        bool mine = lt >= lo && lt < hi;
-        if (by_group) {
-          const int64_t p_lo = (int64_t)lo * p.nRt, p_hi = (int64_t)hi * p.nRt;
-          mine = pid >= p_lo && pid < p_hi;
-          if (mine) {
-            const int nl = hi - lo;
-            const int64_t pe = pid - p_lo, width = (int64_t)GL * nl;
-            const int first_r = (int)(pe / width) * GL;
-            const int gsz = p.nRt - first_r < GL ? p.nRt - first_r : GL;
-            const int in_grp = (int)(pe % width);
-            look.rt = first_r + in_grp % gsz;
-            my_lt = lo + in_grp / gsz;
+      g = p.E;
+      l0 = 0;
+      lvalid = 0;
+      for (int base = 0; base < p.E; base += 64) {
+        if (base > 0) {  // more than 64 groups: the next 64
+          const int e = base + lane;
+          t_lo = t_hi = 0;
+          if (e < p.E) {
+            t_lo = p.tile_off[e];
+            t_hi = p.tile_off[e + 1];
+            r_lo = p.goff[e];
+            r_hi = p.goff[e + 1];
           }
         }
-        if (mine) {
-          const int64_t first = rows_lo + (int64_t)(my_lt - lo) * BM, left = rows_hi - first;
-          look.g = e;
-          look.l0 = first;
-          look.lvalid = left < BM ? (int)left : BM;
+        int my_lt = lt, my_rt = 0;
+        bool mine = lt >= t_lo && lt < t_hi;  // empty groups (and lanes past E) hold no tile
+        if (by_group) {
+          const int64_t p_lo = (int64_t)t_lo * p.nRt, p_hi = (int64_t)t_hi * p.nRt;
+          mine = pid >= p_lo && pid < p_hi;
+          const int nl = mine ? t_hi - t_lo : 1;
+          const int64_t pe = pid - p_lo, width = (int64_t)GL * nl;
+          const int first_r = (int)(pe / width) * GL;
+          const int gsz = p.nRt - first_r < GL ? p.nRt - first_r : GL;
+          const int in_grp = (int)(pe % width);
+          my_rt = first_r + in_grp % (gsz > 0 ? gsz : 1);
+          my_lt = t_lo + in_grp / (gsz > 0 ? gsz : 1);
         }
-      };
-      if (tid < p.E) claim(tid, t_lo, t_hi, r_lo, r_hi);
-      for (int e = tid + NT; e < p.E; e += NT) claim(e, p.tile_off[e], p.tile_off[e + 1], p.goff[e], p.goff[e + 1]);
-      __syncthreads();
-      g = look.g;
+        const unsigned long long hit = __ballot(mine);
+        if (hit != 0) {  // exactly one group holds the tile
+          const int src = __builtin_ctzll(hit);
+          const int64_t first = r_lo + (int64_t)(my_lt - t_lo) * BM, left = r_hi - first;
+          const int lv = left < BM ? (int)left : BM;
+          g = base + src;
+          l0 = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)((uint64_t)first >> 32), src) << 32) |
+                         (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(uint64_t)first, src));
+          lvalid = __builtin_amdgcn_readlane(lv, src);
+          if (by_group) rt = __builtin_amdgcn_readlane(my_rt, src);
+          break;
+        }
+      }
       if (g >= p.E) return;
-      l0 = look.l0;
-      lvalid = look.lvalid;
-      if (by_group) rt = look.rt;
     } else {
       g = 0;
       l0 = (int64_t)lt * BM;
