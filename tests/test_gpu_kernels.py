@@ -652,3 +652,71 @@ def test_grouped_gemm_more_groups_than_threads(oracle, dev, M, N, K, E):
             ref[off : off + m] = xd[off : off + m] @ oracle.torch_dequant_block(qw[e].cpu().view(torch.uint8), sw[e].cpu()).double().t()
         off += m
     assert rel_err(y, ref.float()) <= GEMM_TOL_F32
+
+
+def test_grouped_gemm_random_shapes(dev):
+    """Seeded sweep over ragged shapes (both tile configurations, empty groups, partial tiles on both
+    sides, bias, both output types; wgrad with and without accumulation on the same routing) against
+    the definition of the GEMM evaluated in float64 on the device: dequantise, multiply, add."""
+    import random
+
+    from atorch_amd import kernels
+
+    rnd = random.Random(11)
+
+    def deq_tile(q, s):
+        return q.float() * s.repeat_interleave(TILE, -1)
+
+    def deq_block(q, s):
+        return q.float() * s.repeat_interleave(TILE, -2).repeat_interleave(TILE, -1)
+
+    for case in range(12):
+        E = rnd.choice([1, 2, 3, 5, 8, 17, 64, 130])
+        N = TILE * rnd.choice([1, 2, 3, 4, 5, 8, 11])
+        K = TILE * rnd.choice([1, 2, 3, 4, 8, 9])
+        M = rnd.randint(1, 3000) if case % 2 else rnd.randint(20000, 40000)
+        cuts = sorted(rnd.randint(0, M) for _ in range(E - 1))
+        if E > 3:
+            cuts[1] = cuts[0]  # an empty group
+        b = [0] + cuts + [M]
+        splits = [b[i + 1] - b[i] for i in range(E)]
+        x = randn_bf16((M, K), 100 + case).to(dev)
+        w = randn_bf16((E, N, K), 200 + case, std=0.02).to(dev)
+        qx, sx = kernels.tile_quant(x)
+        qw, sw, _, _ = kernels.block_quant_batched(w)
+        goff = kernels.group_offsets_from_splits(splits, dev)
+        bias = randn_bf16((E, N), 300 + case).to(dev) if case % 3 == 0 else None
+        odt = torch.bfloat16 if case % 4 < 2 else torch.float32
+        y = kernels.grouped_gemm_nt(qx, sx, qw, sw, goff, out_dtype=odt, bias=bias)
+        xd = deq_tile(qx, sx).double()
+        ref = torch.zeros(M, N, dtype=torch.float64, device=dev)
+        off = 0
+        for e, m in enumerate(splits):
+            if m:
+                ref[off : off + m] = xd[off : off + m] @ deq_block(qw[e], sw[e]).double().t()
+                if bias is not None:
+                    ref[off : off + m] += bias[e].double()
+            off += m
+        tol = GEMM_TOL if odt == torch.bfloat16 else GEMM_TOL_F32
+        assert rel_err(y.cpu(), ref.float().cpu()) <= tol, (case, M, N, K, E)
+        if N * K * E > 32 * 1024 * 1024:
+            continue
+        dy = randn_bf16((M, N), 400 + case, std=1e-2).to(dev)
+        _, _, qxt, sxt = kernels.tile_quant_dual_grouped(x, goff, E, rowwise=False)
+        _, _, qdt, sdt = kernels.tile_quant_dual_grouped(dy, goff, E, ld_t=qxt.shape[1], rowwise=False)
+        base = torch.randn(E, N, K, generator=torch.Generator().manual_seed(case)).to(dev)
+        acc = base.clone()
+        kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out=acc, accumulate=True)
+        dw = kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out_dtype=torch.float32)
+        refw = torch.zeros(E, N, K, dtype=torch.float64, device=dev)
+        pos = 0
+        for e, m in enumerate(splits):
+            pad = (m + TILE - 1) // TILE * TILE
+            if m:
+                a = qdt[:, pos : pos + pad].float() * sdt[pos // TILE : (pos + pad) // TILE].t().repeat_interleave(TILE, 1)
+                c = qxt[:, pos : pos + pad].float() * sxt[pos // TILE : (pos + pad) // TILE].t().repeat_interleave(TILE, 1)
+                refw[e] = a.double() @ c.double().t()
+            pos += pad
+        assert rel_err(dw.cpu(), refw.float().cpu()) <= GEMM_TOL_F32, (case, M, N, K, E)
+        # the sum with the old values rounds once more in fp32
+        assert rel_err((acc - base).cpu(), refw.float().cpu()) <= 4 * GEMM_TOL_F32, (case, M, N, K, E)
