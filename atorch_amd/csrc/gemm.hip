@@ -26,6 +26,7 @@
 // are XOR-swizzled so that the linear 1 KB writes of the direct loads and the 32-row MFMA
 // operand reads are both bank-conflict free on the 64-bank LDS (measured: ~235 of 256 B/clk).
 #include <stdlib.h>
+#include <string.h>
 
 #include "common.hpp"
 
@@ -112,13 +113,7 @@ struct Cfg {
   static_assert((NT / 8) % 16 == 0, "the swizzle of a slab depends on the wave only");
 };
 typedef Cfg<2, 2, 2, 2, 3> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two workgroups per CU
-#ifndef AAMD_LARGE_PRB
-#define AAMD_LARGE_PRB 1
-#endif
-#ifndef AAMD_LARGE_LAHEAD
-#define AAMD_LARGE_LAHEAD true
-#endif
-typedef Cfg<2, 4, 4, 2, AAMD_LARGE_PRB, AAMD_LARGE_LAHEAD> CfgLarge;  // 512 threads, 256 (L) x 256 (R); one product buffer: 256 registers per lane
+typedef Cfg<2, 4, 4, 2, 1, true> CfgLarge;  // 512 threads, 256 (L) x 256 (R); one product buffer: 256 registers per lane
 typedef Cfg<2, 4, 2, 2> CfgWgrad;  // 512 threads, 256 (L) x 128 (R): room for the per-row R scales
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
@@ -164,16 +159,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   float* const LsB0 = Sc1 + NT;  // scale batches (kRaggedRows)
 
   const int tid = threadIdx.x;
-#ifdef AAMD_GEMM_TIMING
-  // measurement build: six time stamps per workgroup go where the bias would be read from
-  // (plus the constant-rate clock at both ends of the workgroup and the hardware ids of the compute unit)
-  unsigned long long stamp[8];
-  stamp[0] = __builtin_readcyclecounter();
-  stamp[6] = __builtin_amdgcn_s_memrealtime();
-#define AAMD_STAMP(i) stamp[i] = __builtin_readcyclecounter(); if (i == 4) stamp[7] = (unsigned long long)__builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11)) | ((unsigned long long)__builtin_amdgcn_s_getreg((20) | (0 << 6) | (31 << 11)) << 32)
-#else
-#define AAMD_STAMP(i)
-#endif
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
   const int lane = tid & 63;
 
@@ -231,14 +216,12 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       lt = first + in_grp % gsz;
       rt = in_grp / gsz;
     }
-#if defined(AAMD_GEMM_ABLATE) && (AAMD_GEMM_ABLATE == 3 || AAMD_GEMM_HOT == 1)
-    lt = 0; rt = 0;  // measurement build: every workgroup streams the same tile
-#endif
   }
 
   int64_t l0;     // first L row of the tile
   int lvalid;     // valid L rows in the tile
   int kb0, nkb;   // contraction blocks [kb0, kb0 + nkb)
+  bool short_operands = false;
   if constexpr (MODE == kRaggedRows) {
     if (p.goff) {
       // exactly one group holds tile lt (empty groups hold none)
@@ -302,10 +285,14 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     lvalid = left < BM ? (int)left : BM;
     kb0 = p.tile_off[g];
     nkb = p.tile_off[g + 1] - kb0;
-    if (kb0 + nkb > p.max_kb) nkb = p.max_kb > kb0 ? p.max_kb - kb0 : 0;  // never read past the buffers
+    // Operand buffers too short for the padded token count (ld_t below the device-side total): never
+    // read past them, and make the failure visible: the group's gradient tile is written as NaN.
+    if (kb0 + nkb > p.max_kb) {
+      nkb = 0;
+      short_operands = true;
+    }
   }
   g = __builtin_amdgcn_readfirstlane(g);
-  AAMD_STAMP(1);
   const int64_t r0 = (int64_t)rt * BN;
   const int64_t rleft = p.Rrows - r0;
   const int rvalid = rleft < BN ? (int)rleft : BN;  // a multiple of 128
@@ -313,11 +300,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // uniform tile bases + per-thread 32-bit offsets
   const uint8_t* Lbase = p.L + uniform_i64(l0 * p.ldl + (int64_t)kb0 * kBK);
   const uint8_t* Rbase = p.R + uniform_i64((int64_t)g * p.r_group_stride + r0 * p.ldr + (int64_t)kb0 * kBK);
-#if defined(AAMD_GEMM_HOT) && AAMD_GEMM_HOT == 2
-  Lbase = p.L;  // measurement build: every workgroup streams the same L tile
-#elif defined(AAMD_GEMM_HOT) && AAMD_GEMM_HOT == 3
-  Rbase = p.R;  // measurement build: every workgroup streams the same R tile
-#endif
   const float* Lsg = p.Ls + (int64_t)kb0 * p.ls_blk_stride;
   const float* Rsg = p.Rs + (int64_t)g * p.rs_group_stride + (int64_t)kb0 * p.rs_blk_stride;
 
@@ -377,11 +359,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // so no VGPR is ever written behind the compiler's back.
   auto lds_addr = [](const void* q) { return (uint32_t)(uintptr_t)(lds_ptr_t)q; };
   const uint32_t soff_b = soff * 4u;
-#ifdef AAMD_GEMM_NOSCALE
-  constexpr int kScaleLd = 0;  // measurement build: no scale loads
-#else
   constexpr int kScaleLd = 1;
-#endif
   // L scales of a row-major [rows, K/128] operand: one 4-byte value per row and step would touch
   // as many cache lines as the tile itself.  Instead 32 bytes per row (eight contraction blocks)
   // are fetched every eighth step, 16 bytes per thread, into [row][8] floats.  The last batch is
@@ -401,8 +379,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   };
   auto dma_scale = [&](int kb, float* Sd) {
     const uint8_t* sb = reinterpret_cast<const uint8_t*>(sbase + (int64_t)kb * s_step);
-    if constexpr (kScaleLd)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
                    ::"v"(soff_b), "s"(sb), "s"(lds_addr(Sd) + (uint32_t)(wave * 256))
                    : "memory");
   };
@@ -451,9 +428,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   };
   // End of a step: this thread's loads have landed, then the workgroup barrier.
   auto dma_wait_and_sync = [&]() {
-#if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE >= 4
-    return;  // measurement build: no waits, no barriers
-#endif
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
 
@@ -501,7 +475,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #pragma unroll
     for (int j = 0; j < C::WTL; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; r++) acc[i][j][r] = short_operands ? __builtin_nanf("") : 0.f;
 
   // One 128-deep step on the stage (Lt, Rt, Sct).  Per 32x32 sub-tile t: two chained MFMAs, then
   // the 16 scale-and-accumulate FMAs of sub-tile t-1 run in their shadow.  The wanted issue
@@ -520,9 +494,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     // fragment of sub-tile row `sub` (32 rows each) of one side, K half h
     typedef const __attribute__((address_space(3))) v4i* lds_v4i_t;
     auto load_frag = [&](const uint32_t (&base)[2][2], int rows_per_stage, int sub, int h) {
-#if defined(AAMD_GEMM_ABLATE) && AAMD_GEMM_ABLATE >= 5
-      { v8i f; asm volatile("" : "=v"(f)); return f; }  // measurement build: operands from nowhere
-#endif
       const uint32_t delta = (uint32_t)((stage * rows_per_stage + sub * 32) * kBK);
       const v4i lo = *(lds_v4i_t)(uintptr_t)(base[h][0] + delta);
       const v4i hi = *(lds_v4i_t)(uintptr_t)(base[h][1] + delta);
@@ -620,15 +591,6 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // Measurement builds only: AAMD_GEMM_ABLATE=1 issues no loads inside the loop, =2 skips the MFMA
-  // work, to time the two halves of the pipeline separately.  Results are wrong in both.
-#ifndef AAMD_GEMM_ABLATE
-#define AAMD_GEMM_ABLATE 0
-#endif
-#ifndef AAMD_GEMM_HOT
-#define AAMD_GEMM_HOT 0
-#endif
-  constexpr bool kLoads = AAMD_GEMM_ABLATE != 1 && AAMD_GEMM_ABLATE < 4, kMath = AAMD_GEMM_ABLATE < 2 || AAMD_GEMM_ABLATE >= 4;
   auto nothing = [] {};
   auto no_feed = [](auto) {};
   // Two workgroups per CU: the loads of a step go out in one burst after the barrier (issued a few
@@ -639,13 +601,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     // a wave without valid rows runs its own copy of the loop, loads and barriers only
     auto loop = [&](auto W) {
-      constexpr bool kWork = kMath && decltype(W)::value;
+      constexpr bool kWork = decltype(W)::value;
       int kb = 0;
       for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
-        if (kLoads) dma(kb + 1, Lbuf1, Rbuf1, Sc1);
+        dma(kb + 1, Lbuf1, Rbuf1, Sc1);
         if constexpr (kWork) compute(kb, 0, Sc0, nothing, no_feed);
         dma_wait_and_sync();
-        if (kLoads) dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
+        dma(kb + 2 < nkb ? kb + 2 : kb + 1, Lbuf0, Rbuf0, Sc0);  // the last prefetch re-reads a valid block
         if constexpr (kWork) compute(kb + 1, 1, Sc1, nothing, no_feed);
         dma_wait_and_sync();
       }
@@ -661,97 +623,60 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     // Loads complete in issue order, so "all but the newest L group" is one wait count.  Past the
     // end the loads re-read the last block to keep the counts uniform.
     auto kclamp = [&](int k) { return k < nkb ? k : nkb - 1; };
-#ifdef AAMD_GEMM_BARSTAT
-    // measurement build: cycles this wave spends waiting for its loads, in the end-of-step barrier
-    // and in the mid-step barrier
-    unsigned long long bs_load = 0, bs_end = 0, bs_mid = 0;
-    auto wait_all_but_newest_l = [&]() {
-      const unsigned long long t0 = __builtin_readcyclecounter();
-      if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(C::LCH + kScaleLd) : "memory");
-      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(C::LCH) : "memory");
-      const unsigned long long t1 = __builtin_readcyclecounter();
-      asm volatile("s_barrier" ::: "memory");
-      const unsigned long long t2 = __builtin_readcyclecounter();
-      bs_load += t1 - t0;
-      bs_end += t2 - t1;
-    };
-#else
     auto wait_all_but_newest_l = [&]() {
       if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
       else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
     };
-#endif
     if (nkb > 0) {
       dmaL(0, Lbuf0, Sc0);
       dmaR(0, Rbuf0, Sc0);
       dmaL(kclamp(1), Lbuf1, Sc1);
-      AAMD_STAMP(2);
       wait_all_but_newest_l();
-      AAMD_STAMP(3);
       // a wave without valid rows runs its own copy of the loop, loads and barriers only
       auto loop = [&](auto W) {
-      constexpr bool kWork = decltype(W)::value;
-      auto step = [&](int kb, int stage, uint8_t* Lc, float* Sc, uint8_t* Rn, float* Sn) {
-        // One workgroup per CU: a burst of loads right after the barrier holds up every wave's first
-        // MFMAs, so the tile loads go out a few at a time behind the first sub-tiles (measured 4-5 %
-        // faster): the R tile before the barrier that frees the L half, the L tile after it.  The
-        // scale loads sit behind uniform branches and stay at the head of their group: control flow
-        // inside the sub-tile sequence costs the register allocator dearly.
-        constexpr int RT = C::WTL, RPER = C::RCH / RT;
-        static_assert(C::RCH % RT == 0 && RT + C::LCH <= NTILES, "spread schedule");
-        const int kr = kclamp(kb + 1), kl = kclamp(kb + 2);
-        auto mid = [&]() {
-#ifdef AAMD_GEMM_BARSTAT
-          const unsigned long long t0 = __builtin_readcyclecounter();
-#endif
-          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
-#ifdef AAMD_GEMM_BARSTAT
-          bs_mid += __builtin_readcyclecounter() - t0;
-#endif
-          if (kLoads && !kMath) dmaL(kl, Lc, Sc);
-          else if (kLoads) dmaL_scales(kl, Sc);
-        };
-        auto feed = [&](auto T) {
-          constexpr int t = decltype(T)::value;
-          if (!kLoads) return;
-          if constexpr (t < RT) {
-            static_for<RPER>([&](auto N) { dmaR_tile(t * RPER + decltype(N)::value, kr, Rn); });
-          } else if constexpr (t < RT + C::LCH) {
-            dmaL_tile(t - RT, kl, Lc);
+        constexpr bool kWork = decltype(W)::value;
+        auto step = [&](int kb, int stage, uint8_t* Lc, float* Sc, uint8_t* Rn, float* Sn) {
+          // One workgroup per CU: a burst of loads right after the barrier holds up every wave's first
+          // MFMAs, so the tile loads go out a few at a time behind the first sub-tiles (measured 4-5 %
+          // faster): the R tile before the barrier that frees the L half, the L tile after it.  The
+          // scale loads sit behind uniform branches and stay at the head of their group: control flow
+          // inside the sub-tile sequence costs the register allocator dearly.
+          constexpr int RT = C::WTL, RPER = C::RCH / RT;
+          static_assert(C::RCH % RT == 0 && RT + C::LCH <= NTILES, "spread schedule");
+          const int kr = kclamp(kb + 1), kl = kclamp(kb + 2);
+          auto mid = [&]() {
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
+            dmaL_scales(kl, Sc);
+          };
+          auto feed = [&](auto T) {
+            constexpr int t = decltype(T)::value;
+            if constexpr (t < RT) {
+              static_for<RPER>([&](auto N) { dmaR_tile(t * RPER + decltype(N)::value, kr, Rn); });
+            } else if constexpr (t < RT + C::LCH) {
+              dmaL_tile(t - RT, kl, Lc);
+            }
+          };
+          dmaR_scales(kr, Sn);
+          if constexpr (kWork) {
+            compute(kb, stage, Sc, mid, feed);
+          } else {
+            static_for<NTILES>([&](auto T) {
+              feed(T);
+              if (decltype(T)::value == C::WTL - 1) mid();
+            });
           }
+          wait_all_but_newest_l();
         };
-        if (kLoads && !kMath) dmaR(kr, Rn, Sn);
-        else if (kLoads) dmaR_scales(kr, Sn);
-        if constexpr (kMath && kWork) {
-          compute(kb, stage, Sc, mid, feed);
-        } else if constexpr (kMath) {
-          static_for<NTILES>([&](auto T) {
-            feed(T);
-            if (decltype(T)::value == C::WTL - 1) mid();
-          });
-        } else {
-          mid();
+        int kb = 0;
+        for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
+          step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
+          step(kb + 1, 1, Lbuf1, Sc1, Rbuf0, Sc0);
         }
-        if (kLoads) wait_all_but_newest_l();
-        else asm volatile("s_barrier" ::: "memory");
-      };
-      int kb = 0;
-      for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
-        step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
-        step(kb + 1, 1, Lbuf1, Sc1, Rbuf0, Sc0);
-      }
-      if (kb < nkb) step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
+        if (kb < nkb) step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
       };
       if (has_work) loop(std::true_type{});
       else loop(std::false_type{});
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
-#ifdef AAMD_GEMM_BARSTAT
-      if (wave == (int)(blockIdx.x & 7) && lane == 0 && p.bias != nullptr) {
-        unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 8;
-        dst[0] = bs_load; dst[1] = bs_end; dst[2] = bs_mid; dst[3] = __builtin_readcyclecounter() - stamp[3];
-        dst[4] = wave; dst[5] = nkb;
-      }
-#endif
     }
   }
 
@@ -759,8 +684,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // A lane holds, for one output row, groups of four consecutive columns; stored directly that
   // would be 8-byte pieces in 32 different rows per instruction.  Each wave instead transposes its
   // tile through its own LDS region and writes 128-byte row segments: 8 lanes x 16 bytes per row.
-  if (MODE == kRaggedK && nkb == 0 && p.accumulate) return;  // empty group: leave dW untouched
-  AAMD_STAMP(4);
+  if (MODE == kRaggedK && nkb == 0 && p.accumulate && !short_operands) return;  // empty group: leave dW untouched
   __syncthreads();  // every wave is done with the stage buffers
   if (!has_work) return;
   OUT* Cg = reinterpret_cast<OUT*>(p.C) + (int64_t)g * p.c_group_stride;
@@ -872,11 +796,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       __builtin_amdgcn_wave_barrier();  // the next chunk overwrites the region
     }
   };
-#ifdef AAMD_GEMM_TIMING
-  const bool with_bias = false;  // the bias pointer carries the time stamps in that build
-#else
   const bool with_bias = MODE == kRaggedRows && p.bias != nullptr;
-#endif
   auto flush_as = [&](auto tag) {
     if constexpr (MODE == kRaggedRows) {
       if (with_bias) flush(tag, std::true_type{});
@@ -891,25 +811,18 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     if (p.accumulate) flush_as(float{});
     else flush_as(u16{});
   }
-#ifdef AAMD_GEMM_TIMING
-#ifndef AAMD_GEMM_TIMING_PROLOGUE  // that build keeps the group-lookup and loads-issued stamps instead
-  stamp[1] = __builtin_readcyclecounter();  // epilogue issued (overwrites the group-lookup stamp)
-#endif
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  stamp[5] = __builtin_readcyclecounter();
-#ifndef AAMD_GEMM_TIMING_PROLOGUE
-  stamp[2] = __builtin_amdgcn_s_memrealtime();  // constant-rate clock at the end (overwrites the loads-issued stamp)
-#endif
-#ifndef AAMD_GEMM_BARSTAT
-  if (tid == 0 && p.bias != nullptr) {
-    unsigned long long* dst = reinterpret_cast<unsigned long long*>(const_cast<void*>(p.bias)) + blockIdx.x * 8;
-    for (int i = 0; i < 8; i++) dst[i] = stamp[i];
-  }
-#endif
-#endif
 }
 
 int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st);
+
+// Launch options a test or a tuning run may pin (aamd_gemm_set_option); -1 = the library chooses.
+struct GemmOptions {
+  int tile = -1;      // 0: 128x128 tiles, 1: the large configuration
+  int group_r = -1;   // tile order groups R tiles (1) or L tiles (0)
+  int gl = -1;        // tiles that share a panel in the tile order
+  int ls_batch = -1;  // 0: L scales fetched one contraction block at a time
+};
+static GemmOptions g_opt;
 
 template <int MODE, bool R_PER_ROW, typename C>
 static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st) {
@@ -923,9 +836,9 @@ static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st
   if (MODE == kRaggedK) p.group_r = p.nRt > p.nLt;
   else p.group_r = p.goff != nullptr && (int64_t)p.nRt * C::BM * p.E > p.Lrows;
   if (MODE == kRaggedRows && p.group_r) p.gl = 4;
-  // overrides for experiments and tests
-  if (const char* env = getenv("AAMD_GEMM_GROUP_R")) p.group_r = atoi(env) != 0 && (MODE == kRaggedK || p.goff != nullptr);
-  if (const char* env = getenv("AAMD_GEMM_GL")) p.gl = atoi(env) > 0 ? atoi(env) : p.gl;
+  // overrides set through aamd_gemm_set_option
+  if (g_opt.group_r >= 0) p.group_r = g_opt.group_r != 0 && (MODE == kRaggedK || p.goff != nullptr);
+  if (g_opt.gl > 0) p.gl = g_opt.gl;
 
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "grouped_gemm: grid too large");
   dim3 grid((unsigned)blocks), block(C::NT);
@@ -937,12 +850,11 @@ static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st
   return AAMD_OK;
 }
 
-// Large tiles whenever the problem has enough of them to fill the chip; AAMD_GEMM_TILE=small|large overrides.
-// Tile choice.  AAMD_GEMM_TILE=small|large overrides it (for experiments and tests).
+// Tile choice: large tiles whenever the problem has enough of them to fill the chip
+// (option "tile": 0 forces the small configuration, 1 the large one).
 static bool use_large_tiles(int64_t tiles_256, bool by_default) {
-  const char* env = getenv("AAMD_GEMM_TILE");
-  if (env && env[0] == 's') return false;
-  if (env && env[0] == 'l') return true;
+  if (g_opt.tile == 0) return false;
+  if (g_opt.tile == 1) return true;
   // 256x256 tiles halve the bytes every CU pulls from L2 and measured faster wherever the launch
   // still fills the GPU with them; small launches keep the 128x128 tiles (two workgroups per CU).
   return by_default && tiles_256 >= 512;
@@ -954,10 +866,19 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 using namespace aamd;
 
-extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b,
-                                        const float* b_s, int b_tile_scaled, const int64_t* group_offsets, int E,
-                                        int32_t* tile_ws, int64_t M, int64_t N, int64_t K, void* c, int c_dtype,
-                                        int64_t ldc, const void* bias, int bias_dtype, void* stream) {
+extern "C" int aamd_gemm_set_option(const char* name, int value) {
+  AAMD_REQUIRE(name != nullptr, "gemm_set_option: null name");
+  if (!strcmp(name, "tile")) g_opt.tile = value;
+  else if (!strcmp(name, "group_r")) g_opt.group_r = value;
+  else if (!strcmp(name, "gl")) g_opt.gl = value;
+  else if (!strcmp(name, "ls_batch")) g_opt.ls_batch = value;
+  else AAMD_REQUIRE(false, "gemm_set_option: unknown option '%s'", name);
+  return AAMD_OK;
+}
+
+static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b, const float* b_s,
+                        int b_tile_scaled, const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t M, int64_t N,
+                        int64_t K, void* c, int c_dtype, int64_t ldc, const void* bias, int bias_dtype, void* stream) {
   AAMD_REQUIRE(c_dtype == AAMD_BF16 || c_dtype == AAMD_F32, "grouped_gemm_nt: unsupported output dtype %d", c_dtype);
   AAMD_REQUIRE(M >= 0 && N >= 0 && K >= 0, "grouped_gemm_nt: negative size");
   AAMD_REQUIRE(K % kBK == 0 && N % kTile == 0, "grouped_gemm_nt: K=%lld and N=%lld must be multiples of 128",
@@ -969,7 +890,8 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
   if (M == 0 || N == 0) return AAMD_OK;
   AAMD_REQUIRE(a && a_s && b && b_s && c, "grouped_gemm_nt: null pointer");
   AAMD_REQUIRE(lda >= K && lda % 16 == 0 && aligned16(a) && aligned16(b), "grouped_gemm_nt: operands must be 16-byte aligned");
-  AAMD_REQUIRE(ldc >= N && ldc % 4 == 0 && aligned16(c), "grouped_gemm_nt: output must be 16-byte aligned");
+  AAMD_REQUIRE(ldc >= N && (ldc * (c_dtype == AAMD_BF16 ? 2 : 4)) % 16 == 0 && aligned16(c),
+               "grouped_gemm_nt: output rows must be 16-byte aligned");
   AAMD_REQUIRE(K > 0, "grouped_gemm_nt: K must be positive");
   AAMD_REQUIRE(lda < (1LL << 23) && K < (1LL << 23), "grouped_gemm_nt: row stride too large");
   hipStream_t st = (hipStream_t)stream;
@@ -985,7 +907,7 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
   p.L = a; p.ldl = lda; p.Ls = a_s; p.ls_row_stride = K / kBK; p.ls_blk_stride = 1;
   // 16-byte loads of scale batches need aligned rows and whole groups of four blocks
   p.ls_batch = (K / kBK) >= 8 && (K / kBK) % 4 == 0 && (reinterpret_cast<uintptr_t>(a_s) & 15) == 0;
-  if (const char* env = getenv("AAMD_GEMM_LS_BATCH")) p.ls_batch = p.ls_batch && atoi(env) != 0;
+  if (g_opt.ls_batch == 0) p.ls_batch = 0;
   p.R = b; p.ldr = K; p.r_group_stride = N * K;
   p.Rs = b_s;
   p.rs_row_stride = K / kBK; p.rs_blk_stride = 1;
@@ -1002,6 +924,14 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
                          : launch_gemm<kRaggedRows, false, CfgLarge>(p, c_dtype, blocks, st);
   return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgSmall>(p, c_dtype, blocks, st)
                        : launch_gemm<kRaggedRows, false, CfgSmall>(p, c_dtype, blocks, st);
+}
+
+extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b,
+                                        const float* b_s, int b_tile_scaled, const int64_t* group_offsets, int E,
+                                        int32_t* tile_ws, int64_t M, int64_t N, int64_t K, void* c, int c_dtype,
+                                        int64_t ldc, const void* bias, int bias_dtype, void* stream) {
+  return gemm_nt_impl(a, lda, a_s, b, b_s, b_tile_scaled, group_offsets, E, tile_ws, M, N, K, c, c_dtype, ldc, bias,
+                      bias_dtype, stream);
 }
 
 extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt, const uint8_t* xt,

@@ -421,3 +421,21 @@ def unpermute_combine(
 
 def split_views(t: torch.Tensor, splits: Sequence[int]) -> List[torch.Tensor]:
     return list(torch.split(t, list(splits)))
+
+
+class gemm_options:
+    """Context manager that pins launch choices of the grouped GEMMs (``aamd_gemm_set_option``) and
+    restores the library's own choice on exit: ``with gemm_options(tile=1): ...``."""
+
+    def __init__(self, **opts):
+        self.opts = opts
+
+    def __enter__(self):
+        for k, v in self.opts.items():
+            check(lib().aamd_gemm_set_option(k.encode(), int(v)))
+        return self
+
+    def __exit__(self, *exc):
+        for k in self.opts:
+            check(lib().aamd_gemm_set_option(k.encode(), -1))
+        return False

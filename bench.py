@@ -175,6 +175,12 @@ GEMM_WORKLOADS = {
 def run_gemm(args, kernels, dev):
     E, T, k, zipf, shapes, backward, desc = GEMM_WORKLOADS[args.workload]
     idx, _ = routing(T, E, k, dev, zipf_s=zipf)
+    if zipf is not None:
+        # the ragged configuration asks for empty groups: when the draw has none, the rarest expert's
+        # few tokens go to expert 0
+        cnt = torch.bincount(idx.view(-1), minlength=E)
+        if int((cnt == 0).sum()) == 0:
+            idx = torch.where(idx == cnt.argmin(), torch.zeros_like(idx), idx)
     _, _, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
     M = T * k
     layers = [Layer(kernels, M, K, N, E, goff, dev, 10 * i, backward) for i, (K, N) in enumerate(shapes)]

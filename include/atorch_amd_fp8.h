@@ -156,7 +156,7 @@ int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void *dh, int64_t ld_dh, cons
  *   a [M, K] codes (row stride lda bytes), a_s [M, K/128]
  *   b [E, N, K] codes dense, b_s [E, N/128, K/128] (b_tile_scaled == 0) or [E, N, K/128] (!= 0)
  *   group_offsets [E+1] int64 device, or NULL for a single group [0, M] (then E must be 1)
- *   c [M, N] of c_dtype (row stride ldc elements); rows of empty groups are not touched
+ *   c [M, N] of c_dtype (row stride ldc elements, rows 16-byte aligned); rows of empty groups are not touched
  *   bias [E, N] of bias_dtype or NULL (AAMD_NONE); tile_ws: E+1 int32 scratch.
  *   K % 128 == 0, N % 128 == 0.
  */
@@ -174,11 +174,22 @@ int aamd_grouped_gemm_fp8_nt(const uint8_t *a, int64_t lda, const float *a_s, co
  *   dyt [N, ld_t], sdyt [ld_t/128, N]; xt [K, ld_t], sxt [ld_t/128, K]
  *   dw [E, N, K] of dw_dtype (expert stride in elements); an empty group gives zeros,
  *   or leaves dw_g untouched when accumulate != 0.
+ *   ld_t must cover the padded token total sum_g ceil(M_g/128)*128, which only the device knows:
+ *   a group whose tokens lie beyond ld_t gets NaN in its dw_g instead of a wrong finite gradient.
  */
 int aamd_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uint8_t *xt, const float *sxt,
                                 int64_t ld_t, const int64_t *group_offsets, int E, int32_t *tile_ws, int64_t N,
                                 int64_t K, void *dw, int dw_dtype, int64_t expert_stride, int accumulate,
                                 void *stream);
+
+/*
+ * Pins a launch choice of the grouped GEMMs that the library otherwise makes by itself (for tests
+ * and tuning runs; no counterpart in the reference).  value -1 restores the library's choice.
+ *   "tile": 0 = 128x128 tiles, 1 = the large configuration; "group_r": tile order groups R tiles (1)
+ *   or L tiles (0); "gl": tiles sharing a panel in the tile order; "ls_batch": 0 = activation scales
+ *   fetched one contraction block at a time.  Process-wide; not synchronised with running launches.
+ */
+int aamd_gemm_set_option(const char *name, int value);
 
 /*
  * Inverse permutation + weighted combine in one gather-reduce pass:
@@ -231,6 +242,13 @@ int aamd_bias_gather_add(const void *inp, const void *bias, const void *bin_ids,
                          int64_t H, int E, int dtype, void *out, void *stream);
 int aamd_bias_gather_add_bgrad(const void *grad, const void *bin_ids, int ids_are_i64, int64_t T, int64_t H, int E,
                                int dtype, float *bgrad, void *stream);
+
+/*
+ * Shader clock probe (no counterpart in the reference; the benchmark reports the clock the GEMMs
+ * run at): one wavefront spins for about min_cycles shader cycles (at most 2^31) and writes
+ * out[0] = elapsed shader cycles, out[1] = elapsed ticks of the constant 100 MHz clock.
+ */
+int aamd_clock_probe(uint64_t *out, int64_t min_cycles, void *stream);
 
 #ifdef __cplusplus
 }

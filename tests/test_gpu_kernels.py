@@ -471,6 +471,81 @@ def test_fp8_gemm_tile_scaled_b(oracle, dev):
     assert rel_err(c.cpu(), ref) <= GEMM_TOL_F32
 
 
+def _deq_tile(q, s):
+    return q.float() * s.repeat_interleave(TILE, -1)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_fp8_gemm_tile_scaled_b_large_tiles(dev, out_dtype):
+    """NT GEMM whose B carries 1x128 scales (the dense weight-gradient form, scaled_linear.py:431-446)
+    at a size that takes the large-tile configuration with per-row R scales: partial L tile, odd
+    number of 128-row R tiles; against the float64 definition evaluated on the device."""
+    from atorch_amd import kernels
+
+    M, N, K = 4100, 8320, 512
+    a, b = randn_bf16((M, K), 21).to(dev), randn_bf16((N, K), 22, std=0.02).to(dev)
+    qa, sa = kernels.tile_quant(a)
+    qb, sb = kernels.tile_quant(b)
+    ref = _deq_tile(qa, sa).double() @ _deq_tile(qb, sb).double().t()
+    c = kernels.fp8_gemm(qa, sa, qb, sb, dtype=out_dtype)
+    tol = GEMM_TOL if out_dtype == torch.bfloat16 else GEMM_TOL_F32
+    assert rel_err(c.cpu(), ref.float().cpu()) <= tol
+    # the small-tile configuration computes the same sums in the same order
+    with kernels.gemm_options(tile=0):
+        c_small = kernels.fp8_gemm(qa, sa, qb, sb, dtype=out_dtype)
+    assert torch.equal(c, c_small)
+
+
+@pytest.mark.parametrize("tile", [0, 1], ids=["small", "large"])
+def test_grouped_gemm_wgrad_pinned_tile_configurations(dev, tile):
+    """Both tile configurations of the weight-gradient GEMM (the library picks one by shape) on ragged
+    groups with an empty group and partial token tiles, with and without accumulation, against the
+    float64 definition on the device."""
+    from atorch_amd import kernels
+
+    E, N, K = 5, 640, 384
+    splits = [300, 0, 1111, 128, 77]
+    M = sum(splits)
+    x = randn_bf16((M, K), 31).to(dev)
+    dy = randn_bf16((M, N), 32, std=1e-2).to(dev)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    _, _, qxt, sxt = kernels.tile_quant_dual_grouped(x, goff, E, rowwise=False)
+    _, _, qdt, sdt = kernels.tile_quant_dual_grouped(dy, goff, E, ld_t=qxt.shape[1], rowwise=False)
+    base = torch.randn(E, N, K, generator=torch.Generator().manual_seed(3)).to(dev)
+    acc = base.clone()
+    with kernels.gemm_options(tile=tile):
+        dw = kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out_dtype=torch.float32)
+        dw16 = kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out_dtype=torch.bfloat16)
+        kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out=acc, accumulate=True)
+    refw = torch.zeros(E, N, K, dtype=torch.float64, device=dev)
+    pos = 0
+    for e, m in enumerate(splits):
+        pad = (m + TILE - 1) // TILE * TILE
+        if m:
+            a = qdt[:, pos : pos + pad].float() * sdt[pos // TILE : (pos + pad) // TILE].t().repeat_interleave(TILE, 1)
+            c = qxt[:, pos : pos + pad].float() * sxt[pos // TILE : (pos + pad) // TILE].t().repeat_interleave(TILE, 1)
+            refw[e] = a.double() @ c.double().t()
+        pos += pad
+    refw = refw.float().cpu()
+    assert rel_err(dw.cpu(), refw) <= GEMM_TOL_F32
+    assert rel_err(dw16.cpu(), refw) <= GEMM_TOL
+    assert rel_err((acc - base).cpu(), refw) <= 4 * GEMM_TOL_F32
+    assert torch.all(dw[1] == 0) and torch.equal(acc[1], base[1])
+
+
+def test_grouped_gemm_wgrad_short_operand_buffers_give_nan(dev):
+    """ld_t below the padded token total: the groups that do not fit get NaN, never a finite wrong sum."""
+    from atorch_amd import kernels
+
+    E, N, K = 2, 128, 128
+    splits = [128, 128]
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    qt = torch.zeros((N, 128), dtype=torch.uint8, device=dev).view(kernels.FP8)  # room for one token block only
+    st = torch.ones((1, N), dtype=torch.float32, device=dev)
+    dw = kernels.grouped_gemm_wgrad(qt, st, qt, st, goff, out_dtype=torch.float32)
+    assert torch.all(dw[0] == 0) and torch.all(torch.isnan(dw[1]))
+
+
 @pytest.mark.parametrize("M,N,K,E,mult", [(512, 256, 256, 4, 16), (1000, 128, 384, 6, 1), (300, 384, 128, 3, 128)])
 def test_grouped_gemm_nt(oracle, dev, M, N, K, E, mult):
     from atorch_amd import kernels

@@ -57,3 +57,25 @@ def test_dense_linear_recipe_through_ops_module(oracle, dev):
     assert dw is out and rel_err(dw.cpu(), ref["wgrad"][0]) < 5e-4
     q1, s1, n1, n2 = ops.quantize_vector_blockwise(x.to(dev).view(3, 128, K), fp8, 128)
     assert n1 is None and n2 is None and q1.shape == (3, 128, K) and s1.shape == (3, 128, K // 128)
+
+
+@pytest.mark.gpu
+def test_dense_wgrad_through_ops_module_at_a_size_that_takes_large_tiles(dev):
+    """The dense weight gradient dW = dY^T X of the tile/block recipe (scaled_linear.py:431-446) with
+    an 8192 x 4096 weight: both operands 1x128-scaled along the tokens, large-tile configuration;
+    against the float64 definition evaluated on the device."""
+    from atorch_amd import ops
+
+    M, K, N = 2048, 4096, 8192
+    fp8 = torch.float8_e4m3fn
+    x, dy = randn_bf16((M, K), 5).to(dev), randn_bf16((M, N), 6, std=1e-2).to(dev)
+    _, _, qx_t, sx_t = ops.quantize_vector_blockwise(x, fp8, 128, return_transpose=True)
+    _, _, qdy_t, sdy_t = ops.quantize_vector_blockwise(dy, fp8, 128, return_transpose=True)
+    assert qx_t.shape == (K, M) and sx_t.shape == (K, M // 128)
+    dw = ops.fp8_gemm_blockwise(qdy_t, sdy_t, qx_t, sx_t, torch.float32, is_b_1d_scaled=True)
+
+    def deq(q, s):
+        return (q.float() * s.repeat_interleave(128, -1)).double()
+
+    ref = deq(qdy_t, sdy_t) @ deq(qx_t, sx_t).t()
+    assert dw.shape == (N, K) and rel_err(dw.cpu(), ref.float().cpu()) < 5e-4
