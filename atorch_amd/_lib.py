@@ -51,6 +51,10 @@ SIGNATURES = {
         _int,
         [_vp, _vp, _vp, _vp, _i64, _vp, _int, _vp, _i64, _i64, _vp, _int, _i64, _int, _vp],
     ),
+    "aamd_grouped_gemm_fp8_nt_static": (
+        _int,
+        [_vp, _i64, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp],
+    ),
     "aamd_gemm_set_option": (_int, [ctypes.c_char_p, _int]),
     "aamd_clock_probe": (_int, [_vp, _i64, _vp]),
     "aamd_unpermute_combine": (_int, [_vp, _i64, _i64, _vp, _vp, _int, _i64, _int, _vp, _vp]),

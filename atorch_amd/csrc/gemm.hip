@@ -28,6 +28,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "common.hpp"
 
 namespace aamd {
@@ -931,6 +933,48 @@ extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const flo
                                         int32_t* tile_ws, int64_t M, int64_t N, int64_t K, void* c, int c_dtype,
                                         int64_t ldc, const void* bias, int bias_dtype, void* stream) {
   return gemm_nt_impl(a, lda, a_s, b, b_s, b_tile_scaled, group_offsets, E, tile_ws, M, N, K, c, c_dtype, ldc, bias,
+                      bias_dtype, stream);
+}
+
+// The same GEMM for callers that cannot allocate: the tile prefix lives in a file-scope device
+// array, one copy per GPU, whose address is looked up once per device.
+namespace aamd {
+constexpr int kStaticMaxGroups = AAMD_STATIC_MAX_GROUPS;
+static __device__ __align__(256) int32_t scratch[kStaticMaxGroups + 1];
+constexpr int kMaxDevices = 64;
+static std::atomic<int32_t*> g_scratch_ptr[kMaxDevices];
+
+// Device address of this GPU's copy of `scratch` (the array's name is only a host-side handle).
+static int scratch_of_current_device(int32_t** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  AAMD_REQUIRE(dev >= 0 && dev < kMaxDevices, "grouped_gemm_nt_static: device index %d out of range", dev);
+  int32_t* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    AAMD_REQUIRE(ptr != nullptr, "grouped_gemm_nt_static: no device address for the scratch array");
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = ptr;
+  return AAMD_OK;
+}
+}  // namespace aamd
+
+extern "C" int aamd_grouped_gemm_fp8_nt_static(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b,
+                                               const float* b_s, int b_tile_scaled, const int64_t* group_offsets,
+                                               int E, int64_t M, int64_t N, int64_t K, void* c, int c_dtype,
+                                               int64_t ldc, const void* bias, int bias_dtype, void* stream) {
+  AAMD_REQUIRE(E >= 1 && E <= kStaticMaxGroups, "grouped_gemm_nt_static: E=%d exceeds the %d groups the static scratch holds",
+               E, kStaticMaxGroups);
+  int32_t* ws = nullptr;
+  if (group_offsets != nullptr) {
+    const int rc = scratch_of_current_device(&ws);
+    if (rc) return rc;
+  }
+  // the tile prefix is rewritten in full (E + 1 entries) by the first kernel of every call
+  return gemm_nt_impl(a, lda, a_s, b, b_s, b_tile_scaled, group_offsets, E, ws, M, N, K, c, c_dtype, ldc, bias,
                       bias_dtype, stream);
 }
 

@@ -166,6 +166,20 @@ int aamd_grouped_gemm_fp8_nt(const uint8_t *a, int64_t lda, const float *a_s, co
                              int bias_dtype, void *stream);
 
 /*
+ * aamd_grouped_gemm_fp8_nt for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the same arguments without
+ * tile_ws.  No counterpart in the reference.  The E+1 ints of scratch live in a static device array
+ * of the library (AAMD_STATIC_MAX_GROUPS + 1 ints per GPU, held until the process ends); the call
+ * allocates and frees nothing.  E > AAMD_STATIC_MAX_GROUPS is rejected with AAMD_ERR_ARG.  All calls
+ * on one GPU share that array: calls that may overlap on one GPU (different streams) race on it.
+ */
+#define AAMD_STATIC_MAX_GROUPS 4096
+int aamd_grouped_gemm_fp8_nt_static(const uint8_t *a, int64_t lda, const float *a_s, const uint8_t *b,
+                                    const float *b_s, int b_tile_scaled, const int64_t *group_offsets, int E,
+                                    int64_t M, int64_t N, int64_t K, void *c, int c_dtype, int64_t ldc,
+                                    const void *bias, int bias_dtype, void *stream);
+
+/*
  * Grouped weight-gradient GEMM: dW_g[n, k] (+)= sum over the tokens m of group g of
  * dY[m, n] * X[m, k], both operands 1x128-scaled along the tokens (layouts of
  * aamd_quant_1x128_dual_grouped's q_t / s_t).
