@@ -619,66 +619,157 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     if (has_work) loop(std::true_type{});
     else loop(std::false_type{});
   } else {
-    // The L fragments of a step sit in registers for the whole step, so the L half of a stage is
-    // free as soon as every wave has read it: an extra barrier after those reads lets the L tile of
-    // step k+2 start two steps ahead, and only the R tile of step k+1 has a single step to arrive.
+    // One workgroup per CU, eight waves, two per SIMD.  The matrix pipe of a SIMD idles whenever both
+    // of its waves are away from their MFMAs at the same time, which is what a workgroup barrier
+    // followed by LDS reads produces.  So the two barriers of a step stand where register-resident
+    // MFMA work follows them:
+    //   Q (start of step k): every wave holds the L fragments of step k, so the L half of stage k is
+    //     free and the L tile of step k+2 is requested behind the first sub-tiles;
+    //   P (before the last R row of sub-tiles): every wave has read the last fragments of stage k
+    //     and the tiles of step k+1 have landed; behind it the R tile of step k+2 is requested and
+    //     the first fragments of step k+1 are read from the LDS while the last R row, whose operands
+    //     are already in registers, runs on the matrix pipe.  The fragment registers of step k are
+    //     reused as they die, so the prefetch costs no registers.
+    // The fold of the sub-tile in front of a barrier is issued behind it: the wave that arrives last
+    // has just issued its MFMAs, and the one that waited folds while those still run.
     // Loads complete in issue order, so "all but the newest L group" is one wait count.  Past the
     // end the loads re-read the last block to keep the counts uniform.
+    static_assert(!R_PER_ROW, "the two-barrier pipeline is written for block-scaled R operands");
+    static_assert(C::PRB == 1 && C::WTR % 2 == 0 && C::RCH % C::WTL == 0 && C::LCH <= NTILES, "pipeline shape");
+    constexpr int PT = (C::WTR - 1) * C::WTL - 1;  // the sub-tile in front of barrier P
+    constexpr int RPER = C::RCH / C::WTL;
     auto kclamp = [&](int k) { return k < nkb ? k : nkb - 1; };
-    auto wait_all_but_newest_l = [&]() {
-      if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
-      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
+    typedef const __attribute__((address_space(3))) v4i* lds_v4i_t;
+    auto frag = [&](const uint32_t (&base)[2][2], int stage, int rows_per_stage, int sub, int h) {
+      const uint32_t delta = (uint32_t)((stage * rows_per_stage + sub * 32) * kBK);
+      const v4i lo = *(lds_v4i_t)(uintptr_t)(base[h][0] + delta);
+      const v4i hi = *(lds_v4i_t)(uintptr_t)(base[h][1] + delta);
+      return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
     if (nkb > 0) {
       dmaL(0, Lbuf0, Sc0);
       dmaR(0, Rbuf0, Sc0);
       dmaL(kclamp(1), Lbuf1, Sc1);
-      wait_all_but_newest_l();
-      // a wave without valid rows runs its own copy of the loop, loads and barriers only
-      auto loop = [&](auto W) {
-        constexpr bool kWork = decltype(W)::value;
-        auto step = [&](int kb, int stage, uint8_t* Lc, float* Sc, uint8_t* Rn, float* Sn) {
-          // One workgroup per CU: a burst of loads right after the barrier holds up every wave's first
-          // MFMAs, so the tile loads go out a few at a time behind the first sub-tiles (measured 4-5 %
-          // faster): the R tile before the barrier that frees the L half, the L tile after it.  The
-          // scale loads sit behind uniform branches and stay at the head of their group: control flow
-          // inside the sub-tile sequence costs the register allocator dearly.
-          constexpr int RT = C::WTL, RPER = C::RCH / RT;
-          static_assert(C::RCH % RT == 0 && RT + C::LCH <= NTILES, "spread schedule");
-          const int kr = kclamp(kb + 1), kl = kclamp(kb + 2);
-          auto mid = [&]() {
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave holds its L fragments
-            dmaL_scales(kl, Sc);
-          };
-          auto feed = [&](auto T) {
+      dmaR(kclamp(1), Rbuf1, Sc1);
+      // the tiles of step 0 have landed; those of step 1 may still be on their way
+      if (step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + C::RCH + kScaleLd) : "memory");
+      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + C::RCH) : "memory");
+      auto barrier_q = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+      auto barrier_p = [&]() {
+        if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
+      };
+      if (has_work) {
+        v8i lf[C::WTL][2], rf[2][2];
+        float cs[C::WTL], csn[C::WTL], rblkn;
+        float cs_last = 0.f;  // scale of the sub-tile whose fold is still owed (the last one of the step before)
+        v16f pr, zero;
+#pragma unroll
+        for (int r = 0; r < 16; r++) zero[r] = pr[r] = 0.f;
+        // scales of step kb, which sit in stage buffer `stage`: the lane's L row scales and the R block
+        // scale of the wave; their product is formed where it is first needed, not where the reads are issued
+        auto read_scales = [&](int kb, int stage, float (&dst)[C::WTL], float& rblk) {
+          const float* Sct = stage ? Sc1 : Sc0;
+          const int bsel = kb >> 3;
+          const float* Lsc = batch ? LsB0 + (bsel & 1) * (BM * 8) + (kb - batch_start(bsel)) : Sct;
+          const int lsc_stride = batch ? 8 : 1;
+          rblk = Sct[BM + wrow0 / kTile];
+#pragma unroll
+          for (int j = 0; j < C::WTL; j++) dst[j] = Lsc[(wlrow0 + j * 32 + l32) * lsc_stride];
+        };
+        // (the empty volatile statements pin MFMAs and folds between the memory instructions around
+        // them: plain arithmetic is otherwise free to drift past inline assembly)
+        auto fold = [&](int i, int j, float sc) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][j][r] = __builtin_fmaf(pr[r], sc, acc[i][j][r]);
+          asm volatile("" : "+v"(acc[i][j]));
+        };
+        // fragments and scales of step 0
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          lf[0][h] = frag(la, 0, BM, 0, h);
+          rf[0][h] = frag(ra, 0, BN, 0, h);
+        }
+#pragma unroll
+        for (int j = 1; j < C::WTL; j++)
+#pragma unroll
+          for (int h = 0; h < 2; h++) lf[j][h] = frag(la, 0, BM, j, h);
+        read_scales(0, 0, cs, rblkn);
+#pragma unroll
+        for (int j = 0; j < C::WTL; j++) cs[j] *= rblkn;
+        auto step = [&](int kb, auto S) {
+          constexpr int s = decltype(S)::value;
+          uint8_t* const Lc = s ? Lbuf1 : Lbuf0;
+          uint8_t* const Rc = s ? Rbuf1 : Rbuf0;
+          float* const Scur = s ? Sc1 : Sc0;
+          const int k2 = kclamp(kb + 2);
+          __builtin_amdgcn_sched_barrier(0);
+          barrier_q();
+          __builtin_amdgcn_sched_barrier(0);
+          dmaL_scales(k2, Scur);
+          fold(C::WTR - 1, C::WTL - 1, cs_last);  // owed by the step before (adds zero in the first step)
+          static_for<NTILES>([&](auto T) {
             constexpr int t = decltype(T)::value;
-            if constexpr (t < RT) {
-              static_for<RPER>([&](auto N) { dmaR_tile(t * RPER + decltype(N)::value, kr, Rn); });
-            } else if constexpr (t < RT + C::LCH) {
-              dmaL_tile(t - RT, kl, Lc);
+            constexpr int i = t / C::WTL, j = t % C::WTL;
+            __builtin_amdgcn_sched_barrier(0);
+            pr = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
+            pr = mfma_fp8_32x32x64(rf[i & 1][1], lf[j][1], pr);
+            asm volatile("" : "+v"(pr));
+            __builtin_amdgcn_sched_barrier(0);
+            // memory instructions go out while the MFMAs run, ahead of the fold that waits for them
+            if constexpr (t < C::LCH) dmaL_tile(t, k2, Lc);
+            if constexpr (j == 0 && i + 1 < C::WTR) {
+#pragma unroll
+              for (int h = 0; h < 2; h++) rf[(i + 1) & 1][h] = frag(ra, s, BN, i + 1, h);
             }
-          };
-          dmaR_scales(kr, Sn);
-          if constexpr (kWork) {
-            compute(kb, stage, Sc, mid, feed);
-          } else {
-            static_for<NTILES>([&](auto T) {
-              feed(T);
-              if (decltype(T)::value == C::WTL - 1) mid();
-            });
-          }
-          wait_all_but_newest_l();
+            if constexpr (t == PT) {
+              __builtin_amdgcn_sched_barrier(0);
+              barrier_p();
+              __builtin_amdgcn_sched_barrier(0);
+              dmaR_scales(k2, Scur);
+              // row C::WTR - 2 has been consumed: its registers take the first R row of the next step
+#pragma unroll
+              for (int h = 0; h < 2; h++) rf[0][h] = frag(ra, s ^ 1, BN, 0, h);
+              read_scales(kclamp(kb + 1), s ^ 1, csn, rblkn);
+            }
+            if constexpr (t > PT) {
+              constexpr int jn = t - PT - 1;  // == j: this sub-tile was the last user of lf[j]
+              static_for<RPER>([&](auto N) { dmaR_tile(jn * RPER + decltype(N)::value, k2, Rc); });
+#pragma unroll
+              for (int h = 0; h < 2; h++) lf[jn][h] = frag(la, s ^ 1, BM, jn, h);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (t + 1 < NTILES) fold(i, j, cs[j]);
+          });
+          cs_last = cs[C::WTL - 1];
+#pragma unroll
+          for (int j = 0; j < C::WTL; j++) cs[j] = csn[j] * rblkn;
         };
         int kb = 0;
         for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
-          step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
-          step(kb + 1, 1, Lbuf1, Sc1, Rbuf0, Sc0);
+          step(kb, std::integral_constant<int, 0>{});
+          step(kb + 1, std::integral_constant<int, 1>{});
         }
-        if (kb < nkb) step(kb, 0, Lbuf0, Sc0, Rbuf1, Sc1);
-      };
-      if (has_work) loop(std::true_type{});
-      else loop(std::false_type{});
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
+        if (kb < nkb) step(kb, std::integral_constant<int, 0>{});
+        __builtin_amdgcn_sched_barrier(0);
+        fold(C::WTR - 1, C::WTL - 1, cs_last);
+      } else {
+        // a wave without valid rows: loads and barriers only
+        auto step = [&](int kb, uint8_t* Lc, uint8_t* Rc, float* Scur) {
+          const int k2 = kclamp(kb + 2);
+          barrier_q();
+          dmaL(k2, Lc, Scur);
+          barrier_p();
+          dmaR(k2, Rc, Scur);
+        };
+        int kb = 0;
+        for (; kb + 1 < nkb; kb += 2) {
+          step(kb, Lbuf0, Rbuf0, Sc0);
+          step(kb + 1, Lbuf1, Rbuf1, Sc1);
+        }
+        if (kb < nkb) step(kb, Lbuf0, Rbuf0, Sc0);
+      }
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
     }
   }
 
