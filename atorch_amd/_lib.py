@@ -57,6 +57,7 @@ SIGNATURES = {
     ),
     "aamd_gemm_set_option": (_int, [ctypes.c_char_p, _int]),
     "aamd_clock_probe": (_int, [_vp, _i64, _vp]),
+    "aamd_mfma_probe": (_int, [_vp, _int, _int, _int, _vp, _vp, _vp]),
     "aamd_unpermute_combine": (_int, [_vp, _i64, _i64, _vp, _vp, _int, _i64, _int, _vp, _vp]),
     "aamd_moe_preprocess_ws_ints": (_i64, [_i64, _int]),
     "aamd_moe_preprocess": (_int, [_vp, _int, _i64, _int, _vp, _vp, _vp, _vp, _vp]),

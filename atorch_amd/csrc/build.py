@@ -11,7 +11,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["capi.hip", "quant.hip", "permute.hip", "gemm.hip"]
+SOURCES = ["capi.hip", "quant.hip", "permute.hip", "gemm.hip", "probe.hip"]
 LIB = os.path.join(HERE, "libatorch_amd_fp8.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -31,7 +31,7 @@ def _compile(src: str, extra) -> str:
 
 
 def build(verbose: bool = False, extra_flags=()) -> str:
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=5) as ex:
         objs = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
     subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
     if verbose:

@@ -47,6 +47,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--operands", default="random", choices=["random", "zeros"],
+                    help="GEMM workloads: 'zeros' clears the fp8 codes of the activations and weights after set-up; "
+                         "the same launches then draw far less power (not a result, a measurement of the power limit)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="default workload only: skip the c5 quant/permute kernels, the clock and the matrix-pipe probe")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy before the timed region: under "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its known size calibrates the counters")
@@ -60,6 +65,63 @@ def copy_probe(dev):
     torch.cuda.synchronize()
     dst.copy_(src)
     torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------------------------------
+# probes: shader clock under load, matrix pipes from registers
+# ------------------------------------------------------------------------------------------
+def clock_under(fn, dev, cycles=5_000_000):
+    """Shader clock (GHz) read by a one-wave kernel on a second stream while fn()'s kernels run."""
+    from atorch_amd._lib import check, lib
+
+    out = torch.zeros(2, dtype=torch.int64, device=dev)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    fn()
+    fn()
+    with torch.cuda.stream(side):
+        check(lib().aamd_clock_probe(out.data_ptr(), cycles, side.cuda_stream))
+    fn()
+    fn()
+    torch.cuda.synchronize()
+    c, r = out.cpu().tolist()
+    return round(c / max(r, 1) * 0.1, 3)
+
+
+def mfma_probe(kernels, dev, iters=3000):
+    """TFLOP/s of the GEMM's MFMA sequence issued from registers only, for three operand sets."""
+    from atorch_amd._lib import check, lib
+
+    nbytes = 64 * 512 * 12 * 32
+    g = torch.Generator(device=dev).manual_seed(7)
+    q, _ = kernels.tile_quant(torch.randn((nbytes // 128, 128), generator=g, device=dev).to(torch.bfloat16))
+    rnd = torch.randint(0, 255, (nbytes,), generator=g, device=dev, dtype=torch.uint8)
+    rnd = torch.where((rnd & 0x7F) == 0x7F, rnd ^ 1, rnd)  # no NaN codes
+    sets = {"zeros": torch.zeros(nbytes, dtype=torch.uint8, device=dev), "uniform_random_codes": rnd,
+            "quantised_normal": q.view(torch.uint8).reshape(-1).contiguous()}  # fmt: skip
+    wgs = 1024
+    out = torch.empty(wgs * 512, dtype=torch.float32, device=dev)
+    cyc = torch.zeros(1, dtype=torch.int64, device=dev)
+    res = {}
+    for name, ops in sets.items():
+        for fold in (0, 1):
+            st = torch.cuda.current_stream().cuda_stream
+            check(lib().aamd_mfma_probe(ops.data_ptr(), fold, iters, wgs, out.data_ptr(), cyc.data_ptr(), st))
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            check(lib().aamd_mfma_probe(ops.data_ptr(), fold, iters, wgs, out.data_ptr(), cyc.data_ptr(), st))
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b)
+            fl = wgs * 8 * iters * 16 * 131072.0
+            key = name + ("+fold" if fold else "")
+            res[key] = {"TFLOP/s": round(fl / ms / 1e9, 1)}
+            if fold:
+                # with the fold the two waves of a SIMD alternate on its pipe, so the probed wave runs for the
+                # whole of its round (one of wgs/256): its cycle count over that time is the shader clock
+                res[key]["sclk_ghz"] = round(int(cyc.item()) / (ms * 1e6 / (wgs / 256)), 3)
+    return res
 
 
 # ------------------------------------------------------------------------------------------
@@ -185,6 +247,12 @@ def run_gemm(args, kernels, dev):
     M = T * k
     layers = [Layer(kernels, M, K, N, E, goff, dev, 10 * i, backward) for i, (K, N) in enumerate(shapes)]
     counts = (goff[1:] - goff[:-1]).cpu()
+    if args.operands == "zeros":
+        for L in layers:
+            for name in ("qx", "qw", "qx_t", "qw_t", "qdy", "qdy_t"):
+                t = getattr(L, name, None)
+                if t is not None:
+                    t.view(torch.uint8).zero_()
     torch.cuda.synchronize()
 
     nt_timer, wg_timer = Timer(), Timer()
@@ -243,7 +311,8 @@ def run_gemm(args, kernels, dev):
         "flop_per_launch": nt_flops,
     }
     extras = {"tokens_per_expert_min_max": [int(counts.min()), int(counts.max())],
-              "empty_groups": int((counts == 0).sum())}
+              "empty_groups": int((counts == 0).sum()), "operands": args.operands}
+    extras["sclk_ghz_under_forward_gemm"] = clock_under(lambda: layers[0].fwd(kernels), dev)
     if backward:
         wg_ms = wg_timer.ms()
         wg_avg = sum(wg_ms) / len(wg_ms)
@@ -253,7 +322,7 @@ def run_gemm(args, kernels, dev):
                                   "frac": round(wg_flops / (wg_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
 
     cpu = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.operands == "random":
         cpu = cpu_gemm_baseline(layers[0], counts)
     return {
         "metric": "fp8 grouped-GEMM TFLOPS (fwd+bwd)" if backward else "fp8 grouped-GEMM TFLOPS (fwd)",
@@ -416,6 +485,20 @@ def main():
     if args.copy_probe:
         copy_probe(dev)
     res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
+    if args.workload == "c2" and not args.no_extras:
+        # the other half of the metric (quant / permute GB/s) and the two probes ride along in extras
+        torch.cuda.empty_cache()
+        args5 = argparse.Namespace(**{**vars(args), "no_cpu_baseline": True})
+        r5 = run_c5(args5, kernels, dev)
+        pq = r5["roofline"]
+        res["extras"]["c5"] = {
+            "permute_quant": {"GB/s": pq["achieved"], "frac": pq["frac"], "avg_launch_ms": pq["avg_launch_ms"],
+                              "bytes_per_launch": pq["bytes_per_launch"]},
+            "unpermute_combine": r5["extras"]["unpermute_combine"],
+            "tile_quant_plain": r5["extras"]["tile_quant_plain"],
+        }  # fmt: skip
+        torch.cuda.empty_cache()
+        res["extras"]["mfma_probe"] = mfma_probe(kernels, dev)
     out = {
         "metric": res["metric"],
         "value": res["value"],

@@ -264,6 +264,18 @@ int aamd_bias_gather_add_bgrad(const void *grad, const void *bin_ids, int ids_ar
  */
 int aamd_clock_probe(uint64_t *out, int64_t min_cycles, void *stream);
 
+/*
+ * Matrix-pipe probe (no counterpart in the reference; the benchmark reports what the fp8 MFMA pipes
+ * deliver from registers alone, which on this GPU depends on the operand values through the power
+ * limit): `workgroups` workgroups of eight waves issue, `iters` times, the sixteen
+ * v_mfma_f32_32x32x64_f8f6f4 of one 128-deep step of a 128 x 64 wave tile, with the block-scale fold
+ * (16 FMAs per MFMA pair) when fold != 0.  FLOP = workgroups * 8 * iters * 16 * 131072.
+ *   operands: 64 * 512 * 12 * 32 bytes of fp8 codes (any values), 32-byte aligned
+ *   out: workgroups * 512 floats (checksums); cycles[0]: shader cycles one wave spent in the loop.
+ */
+int aamd_mfma_probe(const void *operands, int fold, int iters, int workgroups, float *out, uint64_t *cycles,
+                    void *stream);
+
 #ifdef __cplusplus
 }
 #endif
