@@ -12,8 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libatorch_amd_fp8.so")
 
 OK, ERR_ARG, ERR_HIP = 0, 1, 2
-NONE, BF16, F32 = -1, 0, 1
-ABI_VERSION = 1
+NONE, BF16, F32, F16 = -1, 0, 1, 2
+ABI_VERSION = 2
 
 _lib: Optional[ctypes.CDLL] = None
 
@@ -57,8 +57,11 @@ SIGNATURES = {
     ),
     "aamd_gemm_set_option": (_int, [ctypes.c_char_p, _int]),
     "aamd_clock_probe": (_int, [_vp, _i64, _vp]),
+    "aamd_stream_probe": (_int, [_vp, _vp, _int, _int, _i64, _i64, _vp]),
     "aamd_mfma_probe": (_int, [_vp, _int, _int, _int, _vp, _vp, _vp]),
-    "aamd_unpermute_combine": (_int, [_vp, _i64, _i64, _vp, _vp, _int, _i64, _int, _vp, _vp]),
+    "aamd_unpermute_combine": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _i64, _int, _vp, _vp]),
+    "aamd_permute_rows_scaled": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp, _int, _vp]),
+    "aamd_unpermute_probs_grad": (_int, [_vp, _int, _vp, _int, _i64, _i64, _vp, _i64, _int, _vp, _vp]),
     "aamd_moe_preprocess_ws_ints": (_i64, [_i64, _int]),
     "aamd_moe_preprocess": (_int, [_vp, _int, _i64, _int, _vp, _vp, _vp, _vp, _vp]),
     "aamd_invert_permutation": (_int, [_vp, _i64, _i64, _vp, _vp]),
@@ -97,12 +100,14 @@ def check(rc: int):
         raise RuntimeError(msg)
 
 
-def dtype_code(dt: torch.dtype) -> int:
+def dtype_code(dt: torch.dtype, quantiser_input: bool = False) -> int:
     if dt == torch.bfloat16:
         return BF16
     if dt == torch.float32:
         return F32
-    raise ValueError(f"atorch_amd: unsupported dtype {dt} (bf16 and fp32 are supported)")
+    if dt == torch.float16 and quantiser_input:
+        return F16
+    raise ValueError(f"atorch_amd: unsupported dtype {dt} (bf16 and fp32 are supported; fp16 as quantiser input)")
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:

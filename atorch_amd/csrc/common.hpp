@@ -65,6 +65,13 @@ struct GLUB {
 struct F32 {
   typedef float elem;
 };
+struct F16 {
+  typedef u16 elem;
+};
+// Inputs whose values are bf16 numbers: quotients by the scale of a bf16 maximum may take the
+// checked three-instruction division (see Divider); fp32 and fp16 inputs take the plain one.
+template <typename IN>
+constexpr bool kBf16Values = !std::is_same<IN, F32>::value && !std::is_same<IN, F16>::value;
 
 __device__ __forceinline__ void unpack8(const v4i& raw, float* v) {
 #pragma unroll

@@ -13,11 +13,17 @@ namespace aamd {
 // ---------------------------------------------------------------------------------------
 constexpr int kMaxTopk = 64;
 
-template <int PD>
-__global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __restrict__ y, int64_t M, int H8,
+// YT: element type of the permuted rows (BF16 or F32); the result has the promoted type of rows and
+// probs (fp32 rows, or fp32 probs, give fp32).
+template <typename YT, int PD>
+__global__ __launch_bounds__(256) void unpermute_combine_kernel(const typename YT::elem* __restrict__ y, int64_t M, int H8,
                                                                 const int32_t* __restrict__ row_map,
                                                                 const void* __restrict__ probs, int topk,
                                                                 void* __restrict__ out) {
+  constexpr bool kRowsF32 = std::is_same<YT, F32>::value;
+  constexpr int VL = kRowsF32 ? 4 : 8;                      // elements per 16-byte chunk (H8 counts chunks)
+  constexpr bool kRoundProducts = !kRowsF32 && PD == AAMD_BF16;  // products are bf16 tensors in the reference
+  constexpr bool kOutF32 = kRowsF32 || PD == AAMD_F32;
   __shared__ int srow[kMaxTopk];
   __shared__ float sprob[kMaxTopk];
   const int64_t t = blockIdx.x;
@@ -31,15 +37,15 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
     sprob[threadIdx.x] = pv;
   }
   __syncthreads();
-  const int64_t H = (int64_t)H8 * 8;
+  const int64_t H = (int64_t)H8 * VL;
   for (int c = threadIdx.x; c < H8; c += blockDim.x) {
     // torch's reduction of a strided dimension, which the reference runs: four accumulators, slot j
     // goes to accumulator j mod 4, the total is ((a0 + a1) + a2) + a3
-    float acc[4][8];
+    float acc[4][VL];
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
-      for (int i = 0; i < 8; i++) acc[a][i] = 0.f;
+      for (int i = 0; i < VL; i++) acc[a][i] = 0.f;
     // B gathered rows at a time: their loads are issued together, then folded in slot order.  (A
     // plain loop over the slots compiles to one load in flight per lane.)  Streaming loads: a
     // permuted row is read exactly once.
@@ -54,7 +60,7 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
         // reference multiplies there.
         const int r = __builtin_amdgcn_readfirstlane(srow[j0 + u]);
         const int keep = r < 0 ? 0 : -1;
-        const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)(r < 0 ? 0 : r) * H) + c;
+        const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)(r < 0 ? 0 : r) * H) + c;  // H elements per row
         raw[u] = __builtin_nontemporal_load(src);
 #pragma unroll
         for (int i = 0; i < 4; i++) raw[u][i] &= keep;
@@ -62,19 +68,23 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
       }
 #pragma unroll
       for (int u = 0; u < B; u++) {
-        float v[8];
-        unpack8(raw[u], v);
+        float v[VL];
+        if constexpr (kRowsF32) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) v[i] = __int_as_float(raw[u][i]);
+        } else {
+          unpack8(raw[u], v);
+        }
         // separate multiply and add (no FMA contraction): the reference multiplies, rounds the
         // product to the promoted dtype, then sums
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) {
+        for (int i = 0; i < VL; i += 2) {
           float p0 = v[i], p1 = v[i + 1];
-          if constexpr (PD == AAMD_BF16) {
+          if constexpr (kRoundProducts) {
             const uint32_t pk = pack_bf16x2(v[i] * pv[u], v[i + 1] * pv[u]);
             p0 = __uint_as_float(pk << 16);
             p1 = __uint_as_float(pk & 0xffff0000u);
-          }
-          if constexpr (PD == AAMD_F32) {
+          } else if constexpr (PD != AAMD_NONE) {
             p0 = v[i] * pv[u];
             p1 = v[i + 1] * pv[u];
           }
@@ -94,19 +104,21 @@ __global__ __launch_bounds__(256) void unpermute_combine_kernel(const u16* __res
     } else if (j < topk) {
       batch(integral_constant<int, 1>{}, j, integral_constant<int, 0>{});
     }
-    float tot[8];
+    float tot[VL];
 #pragma unroll
-    for (int i = 0; i < 8; i++) tot[i] = ((acc[0][i] + acc[1][i]) + acc[2][i]) + acc[3][i];
-    if constexpr (PD == AAMD_F32) {
-      float* dst = reinterpret_cast<float*>(out) + t * H + c * 8;
+    for (int i = 0; i < VL; i++) tot[i] = ((acc[0][i] + acc[1][i]) + acc[2][i]) + acc[3][i];
+    if constexpr (kOutF32) {
+      float* dst = reinterpret_cast<float*>(out) + t * H + c * VL;
       // streaming stores: 5 % faster than plain ones here
       __builtin_nontemporal_store(v4f{tot[0], tot[1], tot[2], tot[3]}, reinterpret_cast<v4f*>(dst));
-      __builtin_nontemporal_store(v4f{tot[4], tot[5], tot[6], tot[7]}, reinterpret_cast<v4f*>(dst) + 1);
+      if constexpr (VL == 8) __builtin_nontemporal_store(v4f{tot[4], tot[5], tot[6], tot[7]}, reinterpret_cast<v4f*>(dst) + 1);
     } else {
-      v4i w;
+      if constexpr (VL == 8) {
+        v4i w;
 #pragma unroll
-      for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(tot[2 * i], tot[2 * i + 1]);
-      __builtin_nontemporal_store(w, reinterpret_cast<v4i*>(reinterpret_cast<u16*>(out) + t * H + c * 8));
+        for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(tot[2 * i], tot[2 * i + 1]);
+        __builtin_nontemporal_store(w, reinterpret_cast<v4i*>(reinterpret_cast<u16*>(out) + t * H + c * 8));
+      }
     }
   }
 }
@@ -124,6 +136,97 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const v4i* __restrict
       const int64_t dst = row_map[t * topk + j];
       if (dst >= 0 && dst < M_out) __builtin_nontemporal_store(v, out + dst * chunks + c);
     }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// row permute with a weight per copy and a conversion: out[row_map[t*k+j]] = OUT(x[t] * probs[t, j]).
+// The gradient of the combine with respect to the permuted rows (what autograd makes of the
+// multiply in token_dispatcher.py:156-158: the product in the promoted type, cast to the rows' type).
+// ---------------------------------------------------------------------------------------
+template <typename IN, typename OUT, int PD>
+__global__ __launch_bounds__(256) void permute_rows_scaled_kernel(const typename IN::elem* __restrict__ x, int64_t cols,
+                                                                  const int32_t* __restrict__ row_map, int topk,
+                                                                  const void* __restrict__ probs, int64_t M_out,
+                                                                  typename OUT::elem* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  for (int64_t c = (int64_t)threadIdx.x * 8; c < cols; c += 256 * 8) {
+    float v[8];
+    if constexpr (std::is_same<IN, F32>::value) {
+      const v4f a = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + t * cols + c));
+      const v4f b = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + t * cols + c) + 1);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        v[i] = a[i];
+        v[4 + i] = b[i];
+      }
+    } else {
+      unpack8(__builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + t * cols + c)), v);
+    }
+    for (int j = 0; j < topk; j++) {
+      const int64_t dst = row_map[t * topk + j];
+      if (dst < 0 || dst >= M_out) continue;
+      float pv = 1.f;
+      if constexpr (PD == AAMD_BF16) pv = bf16_bits_to_f32(reinterpret_cast<const u16*>(probs)[t * topk + j]);
+      if constexpr (PD == AAMD_F32) pv = reinterpret_cast<const float*>(probs)[t * topk + j];
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) o[i] = v[i] * pv;
+      if constexpr (std::is_same<OUT, F32>::value) {
+        __builtin_nontemporal_store(v4f{o[0], o[1], o[2], o[3]}, reinterpret_cast<v4f*>(out + dst * cols + c));
+        __builtin_nontemporal_store(v4f{o[4], o[5], o[6], o[7]}, reinterpret_cast<v4f*>(out + dst * cols + c) + 1);
+      } else {
+        v4i w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (int)pack_bf16x2(o[2 * i], o[2 * i + 1]);
+        __builtin_nontemporal_store(w, reinterpret_cast<v4i*>(out + dst * cols + c));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// gradient of the combine with respect to the weights: dprobs[t, j] = <dout[t], y[row_map[t*k+j]]>
+// (fp32 products and sums; one workgroup per token)
+// ---------------------------------------------------------------------------------------
+template <typename DT, typename YT>
+__global__ __launch_bounds__(256) void unpermute_probs_grad_kernel(const typename DT::elem* __restrict__ dout,
+                                                                   const typename YT::elem* __restrict__ y, int64_t M,
+                                                                   int64_t H, const int32_t* __restrict__ row_map,
+                                                                   int topk, float* __restrict__ dprobs) {
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  auto load8 = [&](auto tag, const auto* p, float* v) {
+    using TT = decltype(tag);
+    if constexpr (std::is_same<TT, F32>::value) {
+      const v4f a = *reinterpret_cast<const v4f*>(p), b = *(reinterpret_cast<const v4f*>(p) + 1);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        v[i] = a[i];
+        v[4 + i] = b[i];
+      }
+    } else {
+      unpack8(*reinterpret_cast<const v4i*>(p), v);
+    }
+  };
+  for (int j = 0; j < topk; j++) {
+    const int64_t r = row_map[t * topk + j];
+    float part = 0.f;
+    if (r >= 0 && r < M) {
+      for (int64_t c = (int64_t)threadIdx.x * 8; c < H; c += 256 * 8) {
+        float a[8], b[8];
+        load8(DT{}, dout + t * H + c, a);
+        load8(YT{}, y + r * H + c, b);
+#pragma unroll
+        for (int i = 0; i < 8; i++) part = part + a[i] * b[i];
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+    __syncthreads();
+    if (threadIdx.x == 0) dprobs[t * topk + j] = (red[0] + red[1]) + (red[2] + red[3]);
   }
 }
 
@@ -427,9 +530,10 @@ extern "C" int aamd_bias_gather_add_bgrad(const void* grad, const void* bin_ids,
   return AAMD_OK;
 }
 
-extern "C" int aamd_unpermute_combine(const void* y, int64_t M, int64_t H, const int32_t* row_map,
+extern "C" int aamd_unpermute_combine(const void* y, int y_dtype, int64_t M, int64_t H, const int32_t* row_map,
                                       const void* probs, int probs_dtype, int64_t T, int topk, void* out,
                                       void* stream) {
+  AAMD_REQUIRE(y_dtype == AAMD_BF16 || y_dtype == AAMD_F32, "unpermute_combine: unsupported row dtype %d", y_dtype);
   AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs_dtype == AAMD_BF16 || probs_dtype == AAMD_F32,
                "unpermute_combine: unsupported probs dtype %d", probs_dtype);
   AAMD_REQUIRE(M >= 0 && H >= 0 && T >= 0 && H % 8 == 0, "unpermute_combine: H=%lld must be a multiple of 8",
@@ -441,15 +545,81 @@ extern "C" int aamd_unpermute_combine(const void* y, int64_t M, int64_t H, const
   AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs != nullptr, "unpermute_combine: probs missing");
   AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0, "unpermute_combine: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  const int H8 = (int)(H / 8);
   dim3 grid((unsigned)T), block(256);
-  if (probs_dtype == AAMD_BF16)
-    unpermute_combine_kernel<AAMD_BF16><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
-  else if (probs_dtype == AAMD_F32)
-    unpermute_combine_kernel<AAMD_F32><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
-  else
-    unpermute_combine_kernel<AAMD_NONE><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+  if (y_dtype == AAMD_BF16) {
+    const int H8 = (int)(H / 8);
+    if (probs_dtype == AAMD_BF16)
+      unpermute_combine_kernel<BF16, AAMD_BF16><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+    else if (probs_dtype == AAMD_F32)
+      unpermute_combine_kernel<BF16, AAMD_F32><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+    else
+      unpermute_combine_kernel<BF16, AAMD_NONE><<<grid, block, 0, st>>>((const u16*)y, M, H8, row_map, probs, topk, out);
+  } else {
+    const int H4 = (int)(H / 4);
+    if (probs_dtype == AAMD_BF16)
+      unpermute_combine_kernel<F32, AAMD_BF16><<<grid, block, 0, st>>>((const float*)y, M, H4, row_map, probs, topk, out);
+    else if (probs_dtype == AAMD_F32)
+      unpermute_combine_kernel<F32, AAMD_F32><<<grid, block, 0, st>>>((const float*)y, M, H4, row_map, probs, topk, out);
+    else
+      unpermute_combine_kernel<F32, AAMD_NONE><<<grid, block, 0, st>>>((const float*)y, M, H4, row_map, probs, topk, out);
+  }
   AAMD_LAUNCH_CHECK("unpermute_combine");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_permute_rows_scaled(const void* x, int x_dtype, int64_t T, int64_t cols, const int32_t* row_map,
+                                        int topk, const void* probs, int probs_dtype, int64_t M_out, void* out,
+                                        int out_dtype, void* stream) {
+  AAMD_REQUIRE((x_dtype == AAMD_BF16 || x_dtype == AAMD_F32) && (out_dtype == AAMD_BF16 || out_dtype == AAMD_F32),
+               "permute_rows_scaled: unsupported dtype %d -> %d", x_dtype, out_dtype);
+  AAMD_REQUIRE(!(x_dtype == AAMD_BF16 && out_dtype == AAMD_F32), "permute_rows_scaled: bf16 -> fp32 is not a case of the combine's gradient");
+  AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs_dtype == AAMD_BF16 || probs_dtype == AAMD_F32,
+               "permute_rows_scaled: unsupported probs dtype %d", probs_dtype);
+  AAMD_REQUIRE(T >= 0 && cols >= 0 && cols % 8 == 0, "permute_rows_scaled: cols=%lld must be a multiple of 8", (long long)cols);
+  AAMD_REQUIRE(topk >= 1 && M_out >= 0 && T < 0x7fffffffLL, "permute_rows_scaled: bad topk / sizes");
+  if (T == 0 || cols == 0) return AAMD_OK;
+  AAMD_REQUIRE(x && out && row_map && (probs || probs_dtype == AAMD_NONE), "permute_rows_scaled: null pointer");
+  AAMD_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "permute_rows_scaled: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)T), block(256);
+#define AAMD_PRS(IN_, OUT_, PD_)                                                                                          \
+  permute_rows_scaled_kernel<IN_, OUT_, PD_><<<grid, block, 0, st>>>((const IN_::elem*)x, cols, row_map, topk, probs, M_out, \
+                                                                     (OUT_::elem*)out)
+#define AAMD_PRS_P(IN_, OUT_)                                  \
+  do {                                                         \
+    if (probs_dtype == AAMD_BF16) AAMD_PRS(IN_, OUT_, AAMD_BF16); \
+    else if (probs_dtype == AAMD_F32) AAMD_PRS(IN_, OUT_, AAMD_F32); \
+    else AAMD_PRS(IN_, OUT_, AAMD_NONE);                        \
+  } while (0)
+  if (x_dtype == AAMD_BF16) AAMD_PRS_P(BF16, BF16);
+  else if (out_dtype == AAMD_BF16) AAMD_PRS_P(F32, BF16);
+  else AAMD_PRS_P(F32, F32);
+#undef AAMD_PRS_P
+#undef AAMD_PRS
+  AAMD_LAUNCH_CHECK("permute_rows_scaled");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_unpermute_probs_grad(const void* dout, int dout_dtype, const void* y, int y_dtype, int64_t M, int64_t H,
+                                         const int32_t* row_map, int64_t T, int topk, float* dprobs, void* stream) {
+  AAMD_REQUIRE((dout_dtype == AAMD_BF16 || dout_dtype == AAMD_F32) && (y_dtype == AAMD_BF16 || y_dtype == AAMD_F32),
+               "unpermute_probs_grad: unsupported dtype");
+  AAMD_REQUIRE(M >= 0 && H >= 0 && T >= 0 && H % 8 == 0, "unpermute_probs_grad: H=%lld must be a multiple of 8", (long long)H);
+  AAMD_REQUIRE(topk >= 1 && topk <= kMaxTopk && T < 0x7fffffffLL, "unpermute_probs_grad: bad topk / sizes");
+  if (T == 0) return AAMD_OK;
+  AAMD_REQUIRE(dout && row_map && dprobs && (y || M == 0), "unpermute_probs_grad: null pointer");
+  AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)dout & 15) == 0, "unpermute_probs_grad: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)T), block(256);
+  if (dout_dtype == AAMD_BF16 && y_dtype == AAMD_BF16)
+    unpermute_probs_grad_kernel<BF16, BF16><<<grid, block, 0, st>>>((const u16*)dout, (const u16*)y, M, H, row_map, topk, dprobs);
+  else if (dout_dtype == AAMD_F32 && y_dtype == AAMD_BF16)
+    unpermute_probs_grad_kernel<F32, BF16><<<grid, block, 0, st>>>((const float*)dout, (const u16*)y, M, H, row_map, topk, dprobs);
+  else if (dout_dtype == AAMD_F32 && y_dtype == AAMD_F32)
+    unpermute_probs_grad_kernel<F32, F32><<<grid, block, 0, st>>>((const float*)dout, (const float*)y, M, H, row_map, topk, dprobs);
+  else
+    unpermute_probs_grad_kernel<BF16, F32><<<grid, block, 0, st>>>((const u16*)dout, (const float*)y, M, H, row_map, topk, dprobs);
+  AAMD_LAUNCH_CHECK("unpermute_probs_grad");
   return AAMD_OK;
 }
 

@@ -38,6 +38,21 @@ struct Raw8<F32> {
   }
 };
 
+template <>
+struct Raw8<F16> {
+  v4i a;
+  __device__ __forceinline__ void load(const u16* p, int64_t) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
+  __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v) const {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t w = (uint32_t)a[i];
+      v[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w & 0xffffu));
+      v[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w >> 16));
+    }
+  }
+};
+
 // sigmoid on the hardware transcendental units, one v_exp_f32 and one v_rcp_f32 per value.  Both
 // flush results below the normal range, and 1 / (1 + e^-x) gets there for x below about -87 while
 // x times it is still a normal number, so everything is carried scaled by 2^16 (x r' stays finite for
@@ -139,7 +154,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
                                                           float* __restrict__ s, float eps, int64_t gate_off,
                                                           u16* __restrict__ h_out) {
   // the three-instruction division is checked for bf16 values over scales of bf16 maxima only
-  const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;
+  const bool plain_div = !kBf16Values<IN> || eps != 0.f;
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
   const int64_t base = (int64_t)blockIdx.x * (16 * U);
   const int64_t cols = (int64_t)nt * kTile;
@@ -258,7 +273,7 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
     u16* __restrict__ h_out, const u16* __restrict__ dh = nullptr, int64_t ld_dh = 0) {
-  const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
+  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see quant8
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
   // SwiGLU backward: two teams of 256 threads per workgroup, one for the da tile and one for the db
   // tile of the same features, each with its own staging; both read a and dh at the same time, so
@@ -359,7 +374,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
                                                             uint8_t* __restrict__ q, float* __restrict__ s,
                                                             uint8_t* __restrict__ q_t, float* __restrict__ s_t,
                                                             float eps) {
-  const bool plain_div = sizeof(typename IN::elem) != 2 || eps != 0.f;  // see quant8
+  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see quant8
   __shared__ float part[16];
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
   const int kb = blockIdx.x, nb = blockIdx.y, e = blockIdx.z;
@@ -487,7 +502,7 @@ extern "C" int aamd_quant_1x128(const void* x, int x_dtype, int64_t rows, int64_
 extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
                                         const int32_t* row_map, int topk, int64_t M_out, uint8_t* q, float* s,
                                         float eps, void* stream) {
-  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32, "quant_1x128: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "quant_1x128: unsupported dtype %d", x_dtype);
   AAMD_REQUIRE(T >= 0 && cols >= 0 && cols % kTile == 0, "quant_1x128: cols=%lld must be a multiple of 128",
                (long long)cols);
   AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "quant_1x128: ldx=%lld must be >= cols and a multiple of 8",
@@ -507,11 +522,15 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   if (row_map == nullptr) {
     if (x_dtype == AAMD_BF16)
       quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
+    else if (x_dtype == AAMD_F16)
+      quant_1x128_kernel<F16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
     else
       quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
   } else {
     if (x_dtype == AAMD_BF16)
       quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
+    else if (x_dtype == AAMD_F16)
+      quant_1x128_kernel<F16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
     else
       quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
   }
@@ -523,7 +542,7 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
                                              const int64_t* group_offsets, int E, int32_t* tile_ws, uint8_t* q,
                                              float* s, uint8_t* q_t, float* s_t, int64_t ld_t, float eps,
                                              void* stream) {
-  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32, "quant_dual: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "quant_dual: unsupported dtype %d", x_dtype);
   AAMD_REQUIRE(M >= 0 && cols >= 0 && cols % kTile == 0, "quant_dual: cols=%lld must be a multiple of 128",
                (long long)cols);
   AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "quant_dual: bad ldx=%lld", (long long)ldx);
@@ -547,6 +566,8 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
   const int nt = (int)(cols / kTile);
   if (x_dtype == AAMD_BF16)
     quant_dual_grouped_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
+  else if (x_dtype == AAMD_F16)
+    quant_dual_grouped_kernel<F16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
   else
     quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
   AAMD_LAUNCH_CHECK("quant_dual_grouped");
@@ -635,7 +656,7 @@ extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t 
 extern "C" int aamd_quant_128x128(const void* w, int w_dtype, int64_t E, int64_t N, int64_t K,
                                   int64_t expert_stride, uint8_t* q, float* s, uint8_t* q_t, float* s_t, float eps,
                                   void* stream) {
-  AAMD_REQUIRE(w_dtype == AAMD_BF16 || w_dtype == AAMD_F32, "quant_128x128: unsupported dtype %d", w_dtype);
+  AAMD_REQUIRE(w_dtype == AAMD_BF16 || w_dtype == AAMD_F32 || w_dtype == AAMD_F16, "quant_128x128: unsupported dtype %d", w_dtype);
   AAMD_REQUIRE(E >= 0 && N >= 0 && K >= 0 && N % kTile == 0 && K % kTile == 0,
                "quant_128x128: N=%lld and K=%lld must be multiples of 128", (long long)N, (long long)K);
   AAMD_REQUIRE((q_t == nullptr) == (s_t == nullptr), "quant_128x128: q_t and s_t go together");
@@ -648,6 +669,8 @@ extern "C" int aamd_quant_128x128(const void* w, int w_dtype, int64_t E, int64_t
   dim3 grid((unsigned)(K / kTile), (unsigned)(N / kTile), (unsigned)E), block(256);
   if (w_dtype == AAMD_BF16)
     quant_128x128_kernel<BF16><<<grid, block, 0, st>>>((const u16*)w, expert_stride, N, K, q, s, q_t, s_t, eps);
+  else if (w_dtype == AAMD_F16)
+    quant_128x128_kernel<F16><<<grid, block, 0, st>>>((const u16*)w, expert_stride, N, K, q, s, q_t, s_t, eps);
   else
     quant_128x128_kernel<F32><<<grid, block, 0, st>>>((const float*)w, expert_stride, N, K, q, s, q_t, s_t, eps);
   AAMD_LAUNCH_CHECK("quant_128x128");

@@ -261,6 +261,133 @@ class _ATorchQuantizedGroupedLinear(torch.autograd.Function):
         )
 
 
+def _stack_of(ts) -> Optional[torch.Tensor]:
+    """The equally shaped tensors as one ``[len(ts), ...]`` tensor without a copy when they are dense,
+    equally spaced views of one buffer (the module's weights are); else None."""
+    from .quantization import _base_of_stack
+
+    info = _base_of_stack(list(ts))
+    if info is None or info[1] != ts[0].numel():
+        return None
+    return torch.as_strided(ts[0], (len(ts), *ts[0].shape), (ts[0].numel(), *ts[0].stride()))
+
+
+class _GroupedLinearDeviceOffsets(torch.autograd.Function):
+    """The same three GEMMs driven by device-side ``group_offsets`` (int64 ``[E + 1]``) instead of the
+    host list ``m_splits``: nothing in forward or backward waits for the device, which is what the
+    ``tokens_per_expert.cpu()`` upstream of the reference's call costs (grouped_gemm_moe.py:837).
+    Needs the fused kernels, i.e. the HIP operator; arithmetic, weight cache and gradient
+    conventions are those of ``_ATorchQuantizedGroupedLinear``."""
+
+    @staticmethod
+    def forward(ctx, x, group_offsets, module, is_grad_enabled, is_first_microbatch, *weights_and_biases):
+        from . import kernels
+        from .bias_gather_add import bias_gather_add_bw  # noqa: F401  (used in backward)
+
+        qp = module.qlinear_params
+        E = module.num_gemms
+        weights, biases = weights_and_biases[:E], weights_and_biases[E:]
+        K = weights[0].shape[-1]
+        assert x.shape[-1] == K, "GEMM not possible"
+        assert group_offsets.dtype == torch.int64 and group_offsets.numel() == E + 1 and group_offsets.is_cuda
+        x2d = x.reshape(-1, K).contiguous()
+        out_dtype = x.dtype if qp.mm_fprop.out_dtype is None else qp.mm_fprop.out_dtype
+        kdt = torch.float32 if out_dtype == torch.float16 else out_dtype
+
+        cached = getattr(module, "_stacked_weight_codes", None)
+        update = is_first_microbatch or is_first_microbatch is None or force_quantize_per_microbatch()
+        if update or cached is None or (is_grad_enabled and cached[2] is None):
+            wstack = _stack_of([w.detach() for w in weights])
+            if wstack is None:
+                wstack = torch.stack([w.detach() for w in weights])
+            cached = kernels.block_quant_batched(wstack, eps=qp.w_params.eps, return_transpose=is_grad_enabled)
+            if not force_quantize_per_microbatch():
+                module._stacked_weight_codes = cached
+                for i, cache in enumerate(module.weight_qresult_caches):
+                    cache.data, cache.scale = cached[0][i], cached[1][i]
+                    cache.data_t = cached[2][i] if is_grad_enabled else None
+                    cache.scale_t = cached[3][i] if is_grad_enabled else None
+        qw, sw, qw_t, sw_t = cached
+
+        if is_grad_enabled:
+            qx, sx, qx_t, sx_t = kernels.tile_quant_dual_grouped(x2d, group_offsets, E, eps=qp.x_params.eps)
+        else:
+            qx, sx = kernels.tile_quant(x2d, eps=qp.x_params.eps)
+        bias = None
+        if module.apply_bias:
+            bias = torch.stack([cast_if_needed(b, module.activation_dtype) for b in biases])
+            if bias.dtype == torch.float16:
+                bias = bias.float()
+        out = kernels.grouped_gemm_nt(qx, sx, qw, sw, group_offsets, out_dtype=kdt, bias=bias)
+        if is_grad_enabled:
+            ctx.module, ctx.x_shape, ctx.is_first_microbatch = module, x.shape, is_first_microbatch
+            ctx.weight_refs = list(weights)
+            ctx.num_bias_inputs = len(biases)
+            ctx.fuse_wgrad_accumulation = module.fuse_wgrad_accumulation
+            ctx.save_for_backward(group_offsets, qx_t, sx_t, qw_t, sw_t)
+        return out.to(out_dtype).view(*x.shape[:-1], out.shape[-1])
+
+    @staticmethod
+    def backward(ctx, dy):
+        from . import kernels
+        from .bias_gather_add import bias_gather_add_bw
+
+        goff, qx_t, sx_t, qw_t, sw_t = ctx.saved_tensors
+        module, weights = ctx.module, ctx.weight_refs
+        qp, E = module.qlinear_params, module.num_gemms
+        dy2d = dy.reshape(-1, dy.shape[-1]).contiguous()
+        M = dy2d.shape[0]
+        dgrad_dtype = dy.dtype if qp.mm_dgrad.out_dtype is None else qp.mm_dgrad.out_dtype
+        wgrad_dtype = dy.dtype if qp.mm_wgrad.out_dtype is None else qp.mm_wgrad.out_dtype
+        f32_if_half = lambda dt: torch.float32 if dt == torch.float16 else dt  # noqa: E731
+
+        bgrads = [None] * ctx.num_bias_inputs
+        if module.apply_bias:
+            counts = goff[1:] - goff[:-1]
+            bin_ids = torch.repeat_interleave(torch.arange(E, device=dy.device), counts, output_size=M)
+            g = dy2d if dy2d.dtype != torch.float16 else dy2d.float()
+            bgrads = list(bias_gather_add_bw(g, bin_ids, E).to(dy.dtype).unbind(0))
+        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(dy2d, goff, E, eps=qp.g_params.eps, ld_t=qx_t.shape[1])
+        dgrad = kernels.grouped_gemm_nt(qdy, sdy, qw_t, sw_t, goff, out_dtype=f32_if_half(dgrad_dtype)).to(dgrad_dtype)
+
+        if ctx.is_first_microbatch is not None:
+            accumulate = ctx.fuse_wgrad_accumulation and not ctx.is_first_microbatch
+        else:
+            accumulate = ctx.fuse_wgrad_accumulation
+        if ctx.fuse_wgrad_accumulation:
+            main = _stack_of([w.main_grad for w in weights])
+            if main is not None and main.dtype in (torch.float32, torch.bfloat16):
+                kernels.grouped_gemm_wgrad(qdy_t, sdy_t, qx_t, sx_t, goff, out=main, accumulate=accumulate)
+            else:  # main_grad tensors that do not tile one buffer: one extra pass
+                tmp = kernels.grouped_gemm_wgrad(qdy_t, sdy_t, qx_t, sx_t, goff, out_dtype=torch.float32)
+                for i, w in enumerate(weights):
+                    w.main_grad.add_(tmp[i]) if accumulate else w.main_grad.copy_(tmp[i])
+            wgrads = [w.main_grad for w in weights]
+        else:
+            wbuf = kernels.grouped_gemm_wgrad(qdy_t, sdy_t, qx_t, sx_t, goff, out_dtype=f32_if_half(wgrad_dtype))
+            wgrads = list(wbuf.to(wgrad_dtype).unbind(0))
+        wgrads = [reset_wgrad_if_needed(ctx, w, g) for w, g in zip(weights, wgrads)]
+        return (dgrad.view(ctx.x_shape), None, None, None, None, *wgrads, *bgrads)
+
+
+def patch_grouped_linear(module) -> None:
+    """Registration hook in the shape of ``patch_kitchen_grouped_linear``
+    (quantized_grouped_linear.py:572-584): replaces ``module._QuantizedGroupedLinear`` and
+    ``module.GroupedLinear`` (and, when the module defines them, the reference's own
+    ``_ATorchQuantizedGroupedLinear`` / ``ATorchGroupedLinear`` names) by the classes of this package.
+    ``module`` is ``kitchen.grouped_linear``, ``atorch.modules.fp8.quantized_grouped_linear`` or any
+    namespace a model builds its grouped linears from."""
+    if module is None:
+        return
+    module._QuantizedGroupedLinear = _ATorchQuantizedGroupedLinear
+    module.GroupedLinear = ATorchGroupedLinear
+    for name, cls in (("_ATorchQuantizedGroupedLinear", _ATorchQuantizedGroupedLinear),
+                      ("ATorchGroupedLinear", ATorchGroupedLinear)):  # fmt: skip
+        if hasattr(module, name):
+            setattr(module, name, cls)
+    logger.info("grouped linear of %s patched to the MI355X kernels", getattr(module, "__name__", module))
+
+
 class ATorchGroupedLinear(torch.nn.Module):
     """Applies ``y_i = x_i A_i^T + b_i`` to ``num_gemms`` row groups of one input tensor.
 
@@ -406,10 +533,14 @@ class ATorchGroupedLinear(torch.nn.Module):
     def forward(
         self,
         inp: torch.Tensor,
-        m_splits: List[int],
+        m_splits: Optional[List[int]],
         is_first_microbatch: Optional[bool] = None,
         inp_metas=None,
+        group_offsets: Optional[torch.Tensor] = None,
     ):
+        """``group_offsets`` (not in the reference): exclusive row prefix per group, int64 ``[num_gemms + 1]``
+        on the device, as the dispatcher of this package produces it.  When given, ``m_splits`` may be
+        None and no host copy of the routing is needed."""
         self.set_activation_dtype(inp)
         inp = inp.contiguous()
         assert self.tp_group_initialized, "TP group not initialized"
@@ -418,11 +549,22 @@ class ATorchGroupedLinear(torch.nn.Module):
         assert all(
             isinstance(c, QuantizeResultCache) for c in self.weight_qresult_caches
         ), "weight_qresult_cache must be QuantizeResultCache"
-        assert len(m_splits) == self.num_gemms, "Number of splits should match number of GEMMs."
         assert self.qlinear_params.quantize, "Quantization must be enabled for GroupedLinear"
 
         weight_tensors = [getattr(self, f"weight{i}") for i in range(self.num_gemms)]
         bias_tensors = [getattr(self, f"bias{i}") for i in range(self.num_gemms)]
+
+        if group_offsets is not None:
+            if not getattr(self.qlinear_params.quantize_op, "supports_fused_grouped", False):
+                raise ValueError("group_offsets needs the fused grouped kernels of the HIP operator")
+            fn = _GroupedLinearDeviceOffsets.apply if torch.is_grad_enabled() else _GroupedLinearDeviceOffsets.forward
+            head = () if torch.is_grad_enabled() else (None,)
+            out = fn(*head, inp, group_offsets, self, torch.is_grad_enabled(), is_first_microbatch,
+                     *weight_tensors, *(bias_tensors if self.use_bias else []))  # fmt: skip
+            if self.return_bias:
+                return out, [cast_if_needed(b, self.activation_dtype) for b in bias_tensors]
+            return out
+        assert len(m_splits) == self.num_gemms, "Number of splits should match number of GEMMs."
 
         if torch.is_grad_enabled():
             linear_fn = _ATorchQuantizedGroupedLinear.apply

@@ -74,7 +74,7 @@ def tile_quant(
         return y, s, y_t[:, :rows], s_t.t()
     y = torch.empty(x.shape, dtype=FP8, device=x.device)
     s = torch.empty(*x.shape[:-1], cols // TILE, dtype=torch.float32, device=x.device)
-    check(lib().aamd_quant_1x128(ptr(x), dtype_code(x.dtype), rows, cols, cols, ptr(y), ptr(s), eps, stream()))
+    check(lib().aamd_quant_1x128(ptr(x), dtype_code(x.dtype, True), rows, cols, cols, ptr(y), ptr(s), eps, stream()))
     return y, s
 
 
@@ -144,7 +144,7 @@ def permute_tile_quant(
     s = torch.empty((num_out_rows, cols // TILE), dtype=torch.float32, device=x.device)
     check(
         lib().aamd_permute_quant_1x128(
-            ptr(x), dtype_code(x.dtype), T, cols, cols, ptr(row_map), topk, num_out_rows, ptr(q), ptr(s), eps, stream()
+            ptr(x), dtype_code(x.dtype, True), T, cols, cols, ptr(row_map), topk, num_out_rows, ptr(q), ptr(s), eps, stream()
         )
     )
     return q, s
@@ -191,7 +191,7 @@ def tile_quant_dual_grouped(
     ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
     check(
         lib().aamd_quant_1x128_dual_grouped(
-            ptr(x), dtype_code(x.dtype), M, cols, cols, ptr(group_offsets), num_groups, ptr(ws),
+            ptr(x), dtype_code(x.dtype, True), M, cols, cols, ptr(group_offsets), num_groups, ptr(ws),
             ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, eps, stream(),
         )
     )  # fmt: skip
@@ -301,7 +301,7 @@ def block_quant_batched(w: torch.Tensor, eps: float = 0.0, return_transpose: boo
     estride = w.stride(0) if E > 1 else N * K
     check(
         lib().aamd_quant_128x128(
-            ptr(w), dtype_code(w.dtype), E, N, K, estride, ptr(q), ptr(s), ptr(q_t), ptr(s_t), eps, stream()
+            ptr(w), dtype_code(w.dtype, True), E, N, K, estride, ptr(q), ptr(s), ptr(q_t), ptr(s_t), eps, stream()
         )
     )
     return q, s, q_t, s_t
@@ -403,20 +403,62 @@ def invert_permutation(sorted_indices: torch.Tensor, n_flat: int) -> torch.Tenso
 def unpermute_combine(
     y: torch.Tensor, row_map: torch.Tensor, probs: Optional[torch.Tensor], num_tokens: int, topk: int
 ) -> torch.Tensor:
-    """out[t] = sum_j probs[t,j] * y[row_map[t*topk+j]] in one gather-reduce pass (bf16 rows)."""
-    assert y.dim() == 2 and y.is_contiguous() and y.dtype == torch.bfloat16
+    """out[t] = sum_j probs[t,j] * y[row_map[t*topk+j]] in one gather-reduce pass (bf16 or fp32 rows;
+    the result has the promoted dtype of rows and probs, as the reference's multiply gives it)."""
+    assert y.dim() == 2 and y.is_contiguous() and y.dtype in (torch.bfloat16, torch.float32)
     M, H = y.shape
     assert row_map.dtype == torch.int32 and row_map.numel() == num_tokens * topk
     if probs is None:
-        pd, out_dtype = _lib.NONE, torch.bfloat16
+        pd, out_dtype = _lib.NONE, y.dtype
     else:
         assert probs.shape == (num_tokens, topk)
         probs = probs.contiguous()
         pd = dtype_code(probs.dtype)
-        out_dtype = torch.bfloat16 if probs.dtype == torch.bfloat16 else torch.float32
+        out_dtype = torch.promote_types(y.dtype, probs.dtype)
     out = torch.empty((num_tokens, H), dtype=out_dtype, device=y.device)
-    check(lib().aamd_unpermute_combine(ptr(y), M, H, ptr(row_map), ptr(probs), pd, num_tokens, topk, ptr(out), stream()))
+    check(
+        lib().aamd_unpermute_combine(
+            ptr(y), dtype_code(y.dtype), M, H, ptr(row_map), ptr(probs), pd, num_tokens, topk, ptr(out), stream()
+        )
+    )
     return out
+
+
+def permute_rows_scaled(
+    x: torch.Tensor, row_map: torch.Tensor, topk: int, num_out_rows: int, probs: Optional[torch.Tensor], out_dtype
+) -> torch.Tensor:
+    """out[row_map[t*topk+j]] = (out_dtype)(x[t] * probs[t, j]): the combine's gradient with respect to
+    the permuted rows (rows that no map entry points to are zero)."""
+    assert x.dim() == 2 and x.is_contiguous()
+    T, cols = x.shape
+    assert row_map.dtype == torch.int32 and row_map.numel() == T * topk and row_map.is_contiguous()
+    alloc = torch.empty if num_out_rows == T * topk else torch.zeros  # dropped copies leave rows unwritten
+    out = alloc((num_out_rows, cols), dtype=out_dtype, device=x.device)
+    pd = _lib.NONE if probs is None else dtype_code(probs.dtype)
+    if probs is not None:
+        probs = probs.contiguous()
+    check(
+        lib().aamd_permute_rows_scaled(
+            ptr(x), dtype_code(x.dtype), T, cols, ptr(row_map), topk, ptr(probs), pd, num_out_rows, ptr(out),
+            dtype_code(out_dtype), stream(),
+        )
+    )  # fmt: skip
+    return out
+
+
+def unpermute_probs_grad(dout: torch.Tensor, y: torch.Tensor, row_map: torch.Tensor, topk: int) -> torch.Tensor:
+    """d_probs[t, j] = <dout[t], y[row_map[t*topk+j]]> in fp32."""
+    assert dout.dim() == 2 and dout.is_contiguous() and y.dim() == 2 and y.is_contiguous()
+    T, H = dout.shape
+    assert y.shape[1] == H and row_map.dtype == torch.int32 and row_map.numel() == T * topk
+    dp = torch.empty((T, topk), dtype=torch.float32, device=dout.device)
+    check(
+        lib().aamd_unpermute_probs_grad(
+            ptr(dout), dtype_code(dout.dtype), ptr(y), dtype_code(y.dtype), y.shape[0], H, ptr(row_map), T, topk,
+            ptr(dp), stream(),
+        )
+    )  # fmt: skip
+    return dp
 
 
 def split_views(t: torch.Tensor, splits: Sequence[int]) -> List[torch.Tensor]:

@@ -241,7 +241,7 @@ class HipQuantizeOp:
         s = torch.empty((E, N // TILE, K // TILE), dtype=torch.float32, device=dev)
         q_t = torch.empty((E, K, N), dtype=FP8, device=dev) if return_transpose else None
         s_t = torch.empty((E, K // TILE, N // TILE), dtype=torch.float32, device=dev) if return_transpose else None
-        dt = dtype_code(ws[0].dtype)
+        dt = dtype_code(ws[0].dtype, True)
         if stacked is not None:
             base, estride = stacked
             check(
@@ -284,6 +284,24 @@ class HipQuantizeOp:
         E = len(qa_list)
         assert len(qb_list) == E and len(sa_list) == E and len(sb_list) == E and len(out_list) == E
         if E == 0:
+            return
+        if out_list[0].dtype == torch.float16:
+            # fp16 activations (quantized_grouped_linear.py:533-534): the kernels write fp32 or bf16, so the
+            # GEMM runs into one fp32 buffer laid out like the outputs and is cast once
+            rows = [int(o.shape[0]) for o in out_list]
+            stacked_out = out_list[0].dim() == 2 and all(o.shape[1:] == out_list[0].shape[1:] for o in out_list)
+            assert stacked_out, "fp16 outputs must share their trailing shape"
+            buf = torch.empty((sum(rows), *out_list[0].shape[1:]), dtype=torch.float32, device=out_list[0].device)
+            tmp = list(torch.split(buf, rows))
+            if accumulate:
+                for t, o in zip(tmp, out_list):
+                    t.copy_(o)
+            if bias is not None:
+                bias = [b.float() for b in bias]
+            self.grouped_qgemm(qa_list, qb_list, mm_params, sa_list, sb_list, tmp, bias=bias, accumulate=accumulate,
+                               qparams_x=qparams_x, qparams_w=qparams_w)  # fmt: skip
+            for t, o in zip(tmp, out_list):
+                o.copy_(t)
             return
         w_shape = tuple(qparams_w.quant_tile_shape) if qparams_w is not None else None
         if w_shape is None:

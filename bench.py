@@ -52,6 +52,10 @@ def parse():
                          "the same launches then draw far less power (not a result, a measurement of the power limit)")
     ap.add_argument("--no-extras", action="store_true",
                     help="default workload only: skip the c5 quant/permute kernels, the clock and the matrix-pipe probe")
+    ap.add_argument("--mix-probe", default=None, metavar="R:W[,R:W...]",
+                    help="instead of a workload: GB/s of a pure streaming kernel that reads R and writes W 16-byte "
+                         "words per unit of work (the ceiling of this GPU for a kernel with that mix of bytes); "
+                         "'all' runs every built mix")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy before the timed region: under "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its known size calibrates the counters")
@@ -86,6 +90,41 @@ def clock_under(fn, dev, cycles=5_000_000):
     torch.cuda.synchronize()
     c, r = out.cpu().tolist()
     return round(c / max(r, 1) * 0.1, 3)
+
+
+MIXES = ["1:0", "0:1", "1:1", "2:1", "1:2", "1:4", "4:1", "8:1", "3:2", "2:2"]
+
+
+def mix_probe(dev, mixes, stream_mib=512, iters=5):
+    """GB/s of the streaming probe for each 'R:W' in mixes: R + W streams of stream_mib MiB each."""
+    from atorch_amd._lib import check, lib
+
+    res = {}
+    # streams one after the other, the stride kept off the powers of two: words of equal index in
+    # different streams would otherwise share their DRAM channel and bank
+    stride = (stream_mib << 20) + int(os.environ.get("AAMD_MIX_SKEW", 0x11100))
+    for m in mixes:
+        r, w = (int(v) for v in m.split(":"))
+        src = torch.empty(max(r, 1) * stride, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty(max(w, 1) * stride, dtype=torch.uint8, device=dev)
+        units = (stream_mib << 20) // 16
+        st = torch.cuda.current_stream().cuda_stream
+        call = lambda: check(lib().aamd_stream_probe(src.data_ptr(), dst.data_ptr(), r, w, stride, units, st))  # noqa: E731
+        call()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            call()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / iters
+        nbytes = (r + w) * units * 16
+        gbs = nbytes / ms / 1e6
+        res[m] = {"GB/s": round(gbs, 1), "frac_of_8TBs": round(gbs / PEAK_HBM_GBS, 4), "bytes": nbytes}
+        del src, dst
+        torch.cuda.empty_cache()
+    return res
 
 
 def mfma_probe(kernels, dev, iters=3000):
@@ -484,6 +523,11 @@ def main():
     torch.cuda.set_device(dev)
     if args.copy_probe:
         copy_probe(dev)
+    if args.mix_probe:
+        mixes = MIXES if args.mix_probe == "all" else args.mix_probe.split(",")
+        print(json.dumps({"metric": "streaming probe GB/s by read:write mix", "unit": "GB/s", "n_gpus": 1,
+                          "mixes": mix_probe(dev, mixes)}))  # fmt: skip
+        return
     res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
     if args.workload == "c2" and not args.no_extras:
         # the other half of the metric (quant / permute GB/s) and the two probes ride along in extras

@@ -12,7 +12,9 @@
  *     the message of the last failure on the calling thread;
  *   - fp8 tensors are OCP e4m3fn codes, one byte each; scales are fp32
  *     dequantisation scales  s = max(amax, eps) / 448  (0 -> 1);
- *   - `dtype` arguments: AAMD_BF16 or AAMD_F32 (also AAMD_NONE where stated).
+ *   - `dtype` arguments: AAMD_BF16 or AAMD_F32 (also AAMD_NONE where stated; the inputs of
+ *     aamd_quant_1x128, aamd_permute_quant_1x128, aamd_quant_1x128_dual_grouped and
+ *     aamd_quant_128x128 may also be AAMD_F16).
  *
  * Each entry point names the reference interface it replaces (paths relative
  * to the reference tree root).
@@ -33,8 +35,9 @@ extern "C" {
 #define AAMD_NONE (-1)
 #define AAMD_BF16 0
 #define AAMD_F32 1
+#define AAMD_F16 2 /* accepted as the input type of the quantisers only */
 
-#define AAMD_ABI_VERSION 1
+#define AAMD_ABI_VERSION 2
 
 /* Library identity and error text. */
 int aamd_abi_version(void);
@@ -212,12 +215,28 @@ int aamd_gemm_set_option(const char *name, int value);
  * Each product is rounded to the promoted dtype before the fp32 sum, as the reference's
  * separate multiply and sum do (:156-159); the sum adds in the order of torch's GPU reduction
  * (slot j into accumulator j mod 4, then ((a0 + a1) + a2) + a3).
- *   y [M, H] bf16; row_map [T*topk] int32 (-1 = dropped copy, contributes 0)
- *   probs [T, topk] of probs_dtype (AAMD_BF16 -> out bf16; AAMD_F32 -> out fp32;
- *   AAMD_NONE -> probs ignored, out bf16); H % 8 == 0.
+ *   y [M, H] of y_dtype (bf16 or fp32); row_map [T*topk] int32 (-1 = dropped copy, contributes 0)
+ *   probs [T, topk] of probs_dtype, or AAMD_NONE (probs ignored); out [T, H] has the promoted type of
+ *   rows and probs: bf16 for bf16 rows with bf16 or no probs, fp32 otherwise; H % 8 == 0.
  */
-int aamd_unpermute_combine(const void *y, int64_t M, int64_t H, const int32_t *row_map, const void *probs,
-                           int probs_dtype, int64_t T, int topk, void *out, void *stream);
+int aamd_unpermute_combine(const void *y, int y_dtype, int64_t M, int64_t H, const int32_t *row_map,
+                           const void *probs, int probs_dtype, int64_t T, int topk, void *out, void *stream);
+
+/*
+ * The two gradients of that combine, as autograd derives them from the reference's torch ops
+ * (token_dispatcher.py:155-159: index_copy_, multiply by probs, sum over topk):
+ *   permute_rows_scaled: d_y[row_map[t*topk+j], :] = (out_dtype)(d_out[t, :] * probs[t, j]), the product
+ *     formed in fp32 and rounded once; with probs_dtype == AAMD_NONE it is the plain permute with a
+ *     conversion.  x [T, cols] of x_dtype, out [M_out, cols] of out_dtype (bf16 -> bf16, fp32 -> bf16,
+ *     fp32 -> fp32); cols % 8 == 0; rows no map entry points to are not written.
+ *   unpermute_probs_grad: d_probs[t, j] = sum_h d_out[t, h] * y[row_map[t*topk+j], h] in fp32
+ *     (0 for a dropped copy); d_probs [T, topk] fp32, the caller casts.
+ */
+int aamd_permute_rows_scaled(const void *x, int x_dtype, int64_t T, int64_t cols, const int32_t *row_map, int topk,
+                             const void *probs, int probs_dtype, int64_t M_out, void *out, int out_dtype,
+                             void *stream);
+int aamd_unpermute_probs_grad(const void *dout, int dout_dtype, const void *y, int y_dtype, int64_t M, int64_t H,
+                              const int32_t *row_map, int64_t T, int topk, float *dprobs, void *stream);
 
 /*
  * Router preprocess on the device, no host round trip: histogram of expert ids,
@@ -275,6 +294,16 @@ int aamd_clock_probe(uint64_t *out, int64_t min_cycles, void *stream);
  */
 int aamd_mfma_probe(const void *operands, int fold, int iters, int workgroups, float *out, uint64_t *cycles,
                     void *stream);
+
+/*
+ * Streaming probe (no counterpart in the reference; the benchmark prices the memory-bound kernels
+ * against what the memory system delivers for their mix of read and written bytes): per 16-byte word
+ * of work one word is read from each of `reads` input streams and one written to each of `writes`
+ * output streams, all accesses streaming.  Stream i of src / dst starts at byte i * stride_bytes and
+ * holds `units` words.  Built mixes: 1:0 0:1 1:1 2:1 1:2 1:4 4:1 8:1 3:2 2:2.
+ */
+int aamd_stream_probe(const void *src, void *dst, int reads, int writes, int64_t stride_bytes, int64_t units,
+                      void *stream);
 
 #ifdef __cplusplus
 }

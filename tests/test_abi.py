@@ -64,9 +64,9 @@ def test_argument_validation_without_gpu():
     rc = L.aamd_grouped_gemm_fp8_nt(one, 128, one, one, one, 0, None, 2, None, 8, 128, 128, one, _lib.BF16, 128, None, _lib.NONE, None)
     assert rc == _lib.ERR_ARG and b"group_offsets" in L.aamd_last_error()
     # unpermute: topk out of range, H not a multiple of 8
-    rc = L.aamd_unpermute_combine(one, 8, 64, one, one, _lib.BF16, 4, 100, one, None)
+    rc = L.aamd_unpermute_combine(one, _lib.BF16, 8, 64, one, one, _lib.BF16, 4, 100, one, None)
     assert rc == _lib.ERR_ARG and b"topk" in L.aamd_last_error()
-    rc = L.aamd_unpermute_combine(one, 8, 60, one, one, _lib.BF16, 4, 2, one, None)
+    rc = L.aamd_unpermute_combine(one, _lib.BF16, 8, 60, one, one, _lib.BF16, 4, 2, one, None)
     assert rc == _lib.ERR_ARG
     # preprocess: too many experts
     rc = L.aamd_moe_preprocess(one, 1, 8, 5000, one, one, one, one, None)

@@ -328,3 +328,82 @@ def test_baseline_first_configuration_end_to_end(oracle, dev):
     # does, so the ffn-wide rows go through the kernel wrapper)
     out = kernels.unpermute_combine(y, disp.row_map, probs.to(dev), T, 1)
     assert torch.equal(out.cpu()[sorted_idx], y.cpu())
+
+
+# ------------------------------------------------------------------------------------------
+# boundary: device-side offsets, fp16 activations, registration hook
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_module_with_device_group_offsets_equals_host_splits(dev, bias, fuse):
+    """forward(inp, None, group_offsets=...) runs the same kernels as forward(inp, m_splits): identical
+    outputs and gradients, bit for bit, with bias, fused wgrad accumulation and under no_grad."""
+    from atorch_amd import kernels
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+
+    E, K, N = 5, 256, 384
+    splits = [130, 0, 257, 64, 91]
+    M = sum(splits)
+    torch.manual_seed(4)
+    mods = [ATorchGroupedLinear(E, K, N, bias=bias, params_dtype=torch.bfloat16, device=dev,
+                                fuse_wgrad_accumulation=fuse) for _ in range(2)]  # fmt: skip
+    with torch.no_grad():
+        for i in range(E):
+            mods[1].get_parameter(f"weight{i}").copy_(mods[0].get_parameter(f"weight{i}"))
+            if bias:
+                b = randn_bf16((N,), 80 + i).to(dev)
+                mods[0].get_parameter(f"bias{i}").copy_(b)
+                mods[1].get_parameter(f"bias{i}").copy_(b)
+            if fuse:
+                mg = torch.rand(N, K, generator=torch.Generator().manual_seed(i)).to(dev)
+                mods[0].get_parameter(f"weight{i}").main_grad = mg.clone()
+                mods[1].get_parameter(f"weight{i}").main_grad = mg.clone()
+    x = heavy_tailed((M, K), 21).to(dev)
+    dy = randn_bf16((M, N), 22, std=1e-2).to(dev)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    oa = mods[0](xa, splits)
+    ob = mods[1](xb, None, group_offsets=goff)
+    assert torch.equal(oa, ob)
+    oa.backward(dy)
+    ob.backward(dy)
+    assert torch.equal(xa.grad, xb.grad)
+    for i in range(E):
+        wa, wb = mods[0].get_parameter(f"weight{i}"), mods[1].get_parameter(f"weight{i}")
+        if fuse:
+            assert wa.grad is None and wb.grad is None and torch.equal(wa.main_grad, wb.main_grad)
+        else:
+            assert torch.equal(wa.grad, wb.grad)
+        if bias:
+            ga, gb = mods[0].get_parameter(f"bias{i}").grad, mods[1].get_parameter(f"bias{i}").grad
+            torch.testing.assert_close(ga.float(), gb.float(), rtol=2e-2, atol=1e-4)  # order of an fp32 sum
+    with torch.no_grad():
+        assert torch.equal(mods[1](x, None, group_offsets=goff, is_first_microbatch=False), oa.detach())
+
+
+def test_module_accepts_fp16_activations(dev, oracle):
+    """fp16 inputs and parameters (quantized_grouped_linear.py:533-534): codes and scales come from the fp16
+    values exactly; outputs and gradients are fp16 and within the GEMM tolerance of the oracle."""
+    from atorch_amd import kernels
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+
+    E, K, N = 3, 256, 128
+    splits = [100, 0, 156]
+    torch.manual_seed(5)
+    mod = ATorchGroupedLinear(E, K, N, bias=False, params_dtype=torch.float16, device=dev)
+    x = randn_bf16((sum(splits), K), 31, dtype=torch.float16)
+    dy = randn_bf16((sum(splits), N), 32, std=1e-2, dtype=torch.float16)
+    q, s = kernels.tile_quant(x.to(dev))
+    qo, so = oracle.tile_quant(x.float())
+    assert torch.equal(q.view(torch.uint8).cpu(), qo.view(torch.uint8)) and torch.equal(s.cpu(), so)
+    xg = x.to(dev).requires_grad_(True)
+    out = mod(xg, splits)
+    out.backward(dy.to(dev))
+    assert out.dtype == torch.float16 and xg.grad.dtype == torch.float16
+    ws = [mod.get_parameter(f"weight{i}").detach().float().cpu() for i in range(E)]
+    orc = oracle.grouped_linear_fwd_bwd(x.float(), ws, splits, dy.float())
+    assert rel_err(out.detach().float().cpu(), orc["out"]) <= TOL
+    assert rel_err(xg.grad.float().cpu(), orc["dgrad"]) <= TOL
+    for i in range(E):
+        g = mod.get_parameter(f"weight{i}").grad
+        assert g.dtype == torch.float16 and rel_err(g.float().cpu(), orc["wgrad"][i]) <= TOL

@@ -218,3 +218,16 @@ def test_hip_library_is_required(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(os.path.dirname(_lib.LIB_PATH), "missing.so"))
     with pytest.raises(_lib.HipLibraryMissing):
         _lib.lib()
+
+
+def test_patch_grouped_linear_hook():
+    import types
+
+    from atorch_amd.grouped_linear import ATorchGroupedLinear, _ATorchQuantizedGroupedLinear, patch_grouped_linear
+
+    ns = types.SimpleNamespace(_QuantizedGroupedLinear=object, GroupedLinear=object, ATorchGroupedLinear=object)
+    patch_grouped_linear(ns)
+    assert ns._QuantizedGroupedLinear is _ATorchQuantizedGroupedLinear
+    assert ns.GroupedLinear is ATorchGroupedLinear and ns.ATorchGroupedLinear is ATorchGroupedLinear
+    assert not hasattr(ns, "_ATorchQuantizedGroupedLinear")
+    patch_grouped_linear(None)
