@@ -39,6 +39,11 @@ SIGNATURES = {
         _int,
         [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
     ),
+    "aamd_gelu_quant_1x128": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "aamd_gelu_quant_1x128_dual_grouped": (
+        _int,
+        [_vp, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+    ),
     "aamd_bias_gather_add": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
     "aamd_bias_gather_add_bgrad": (_int, [_vp, _vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
     "aamd_quant_128x128": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _f32, _vp]),

@@ -62,6 +62,16 @@ struct GLU {
 struct GLUB {
   typedef u16 elem;
 };
+// bf16 values x read as h = bf16(gelu(x)), gelu(x) = x/2 (1 + erf(x / sqrt 2)) in fp32: the default
+// activation of the expert MLP (grouped_gemm_moe.py:449, torch.nn.functional.gelu).
+struct GELU {
+  typedef u16 elem;
+};
+// Its backward: values x plus the gradient dh of h (at a fixed element offset from x: both are dense
+// [M, F] tensors); the element read is bf16(dh (cdf(x) + x pdf(x))), autograd's gelu_backward.
+struct GELUB {
+  typedef u16 elem;
+};
 struct F32 {
   typedef float elem;
 };

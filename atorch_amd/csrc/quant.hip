@@ -132,6 +132,52 @@ struct GluBwd8 {
   }
 };
 
+// GELU on load (fp32 arithmetic of the torch op on a bf16 tensor, one rounding to bf16), and its
+// backward dh (cdf + x pdf) with cdf = (1 + erf(x / sqrt 2)) / 2, pdf = exp(-x^2 / 2) / sqrt(2 pi).
+template <>
+struct Raw8<GELU> {
+  v4i a;
+  __device__ __forceinline__ void load(const u16* p, int64_t) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
+  __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v) const {
+    float x[8];
+    unpack8(a, x);
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      const float g0 = x[i] * 0.5f * (1.0f + erff(x[i] * 0.70710678118654752440f));
+      const float g1 = x[i + 1] * 0.5f * (1.0f + erff(x[i + 1] * 0.70710678118654752440f));
+      const uint32_t h = pack_bf16x2(g0, g1);
+      v[i] = __uint_as_float(h << 16);
+      v[i + 1] = __uint_as_float(h & 0xffff0000u);
+    }
+  }
+};
+template <>
+struct Raw8<GELUB> {
+  v4i a, d;
+  __device__ __forceinline__ void load(const u16* p, int64_t dh_off) {
+    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+    d = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p + dh_off));
+  }
+  __device__ __forceinline__ void zero() { a = d = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void get(float* v) const {
+    float x[8], g[8];
+    unpack8(a, x);
+    unpack8(d, g);
+    auto grad = [](float xv, float gv) {
+      const float cdf = 0.5f * (1.0f + erff(xv * 0.70710678118654752440f));
+      const float pdf = 0.39894228040143267794f * __expf(-0.5f * xv * xv);
+      return gv * (cdf + xv * pdf);
+    };
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      const uint32_t h = pack_bf16x2(grad(x[i], g[i]), grad(x[i + 1], g[i + 1]));
+      v[i] = __uint_as_float(h << 16);
+      v[i + 1] = __uint_as_float(h & 0xffff0000u);
+    }
+  }
+};
+
 // 8 values that are bf16-representable -> 16 bytes
 __device__ __forceinline__ v4i pack8_bf16(const float* v) {
   v4i w;
@@ -620,6 +666,61 @@ extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, 
   quant_dual_grouped_kernel<GLU><<<grid, block, 0, st>>>((const u16*)fc1, ld, (int)(F / kTile), group_offsets, tile_ws, E,
                                                          q, s, q_t, s_t, ld_t, 0.f, F, (u16*)h_out);
   AAMD_LAUNCH_CHECK("swiglu_quant_dual_grouped");
+  return AAMD_OK;
+}
+
+// GELU fused into the quantisers: same launches with the GELU / GELU-backward loaders
+extern "C" int aamd_gelu_quant_1x128(const void* x, int64_t rows, int64_t F, int64_t ld, void* h_out, uint8_t* q, float* s,
+                                     void* stream) {
+  AAMD_REQUIRE(rows >= 0 && F >= 0 && F % kTile == 0, "gelu_quant: F=%lld must be a multiple of 128", (long long)F);
+  AAMD_REQUIRE(ld >= F && ld % 8 == 0, "gelu_quant: ld=%lld must be >= F and a multiple of 8", (long long)ld);
+  if (rows == 0 || F == 0) return AAMD_OK;
+  AAMD_REQUIRE(x && q && s, "gelu_quant: null pointer");
+  AAMD_REQUIRE(aligned16(x) && aligned16(q) && aligned16(h_out), "gelu_quant: pointers must be 16-byte aligned");
+  const int nt = (int)(F / kTile);
+  const int64_t total = rows * nt;
+  AAMD_REQUIRE(total < (int64_t)1 << 40, "gelu_quant: too many tiles");
+  constexpr int U = kQuantU;
+  const int64_t blocks = (total + 16 * U - 1) / (16 * U);
+  AAMD_REQUIRE(blocks < 0x7fffffffLL, "gelu_quant: grid too large");
+  quant_1x128_kernel<GELU, false, U><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+      (const u16*)x, ld, nt, total, nullptr, 1, rows, q, s, 0.f, 0, (u16*)h_out);
+  AAMD_LAUNCH_CHECK("gelu_quant_1x128");
+  return AAMD_OK;
+}
+
+// dh == nullptr: forward (h = gelu(x)); else backward (g = dh * gelu'(x)), dh dense with the row stride of x
+extern "C" int aamd_gelu_quant_1x128_dual_grouped(const void* x, const void* dh, int64_t M, int64_t F, int64_t ld,
+                                                  const int64_t* group_offsets, int E, int32_t* tile_ws, void* h_out,
+                                                  uint8_t* q, float* s, uint8_t* q_t, float* s_t, int64_t ld_t,
+                                                  void* stream) {
+  AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "gelu_quant_dual: F=%lld must be a multiple of 128", (long long)F);
+  AAMD_REQUIRE(ld >= F && ld % 8 == 0, "gelu_quant_dual: bad ld=%lld", (long long)ld);
+  AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "gelu_quant_dual: group_offsets / tile_ws required");
+  AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "gelu_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
+  AAMD_REQUIRE((q == nullptr) == (s == nullptr), "gelu_quant_dual: q and s go together");
+  AAMD_REQUIRE(q_t && s_t, "gelu_quant_dual: q_t / s_t required");
+  if (F == 0) return AAMD_OK;
+  const int64_t max_tiles = M / kTile + E;
+  const int64_t grid_tiles = ld_t / kTile < max_tiles ? ld_t / kTile : max_tiles;
+  if (grid_tiles == 0) return AAMD_OK;
+  AAMD_REQUIRE(x != nullptr, "gelu_quant_dual: null input");
+  AAMD_REQUIRE(aligned16(x) && aligned16(dh) && aligned16(q_t) && (!q || aligned16(q)) && aligned16(h_out),
+               "gelu_quant_dual: pointers must be 16-byte aligned");
+  AAMD_REQUIRE(grid_tiles <= 65535, "gelu_quant_dual: more than 65535 token tiles");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
+  if (rc) return rc;
+  dim3 grid((unsigned)(F / kTile), (unsigned)grid_tiles), block(256);
+  if (dh == nullptr) {
+    quant_dual_grouped_kernel<GELU><<<grid, block, 0, st>>>((const u16*)x, ld, (int)(F / kTile), group_offsets, tile_ws, E, q, s,
+                                                            q_t, s_t, ld_t, 0.f, 0, (u16*)h_out);
+  } else {
+    const int64_t dh_off = (const u16*)dh - (const u16*)x;  // elements; the loader reads dh at x + dh_off
+    quant_dual_grouped_kernel<GELUB><<<grid, block, 0, st>>>((const u16*)x, ld, (int)(F / kTile), group_offsets, tile_ws, E, q, s,
+                                                             q_t, s_t, ld_t, 0.f, dh_off, (u16*)h_out);
+  }
+  AAMD_LAUNCH_CHECK("gelu_quant_dual_grouped");
   return AAMD_OK;
 }
 

@@ -288,6 +288,58 @@ def swiglu_bwd_tile_quant_dual_grouped(
     return (q, s, q_t, s_t, g) if return_grad else (q, s, q_t, s_t)
 
 
+def gelu_tile_quant(x: torch.Tensor, return_activation: bool = False):
+    """``h = gelu(x)`` (torch.nn.functional.gelu, the expert MLP's default activation,
+    grouped_gemm_moe.py:449) quantised 1x128 along the last dim without writing ``h``.
+    Returns ``(q, s)`` or ``(q, s, h)``."""
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    F = x.size(-1)
+    assert F % TILE == 0
+    rows = x.numel() // F if F else 0
+    dev = x.device
+    q = torch.empty(x.shape, dtype=FP8, device=dev)
+    s = torch.empty(*x.shape[:-1], F // TILE, dtype=torch.float32, device=dev)
+    h = torch.empty(x.shape, dtype=torch.bfloat16, device=dev) if return_activation else None
+    check(lib().aamd_gelu_quant_1x128(ptr(x), rows, F, F, ptr(h), ptr(q), ptr(s), stream()))
+    return (q, s, h) if return_activation else (q, s)
+
+
+def gelu_tile_quant_dual_grouped(
+    x: torch.Tensor,
+    group_offsets: torch.Tensor,
+    num_groups: int,
+    dh: Optional[torch.Tensor] = None,
+    ld_t: Optional[int] = None,
+    rowwise: bool = True,
+    return_activation: bool = False,
+):
+    """GELU fused into ``tile_quant_dual_grouped``: quantises ``h = gelu(x)`` for ``x [M, F]`` bf16, or,
+    with ``dh [M, F]``, the gradient ``g = dh * gelu'(x)`` (what autograd computes for the activation).
+    Returns ``(q, s, q_t, s_t)`` (plus ``h`` / ``g`` in bf16 with ``return_activation``)."""
+    assert x.dim() == 2 and x.is_contiguous() and x.dtype == torch.bfloat16
+    M, F = x.shape
+    assert F % TILE == 0
+    if dh is not None:
+        assert dh.shape == x.shape and dh.is_contiguous() and dh.dtype == torch.bfloat16
+    assert group_offsets.dtype == torch.int64 and group_offsets.numel() == num_groups + 1
+    if ld_t is None:
+        ld_t = padded_bound(M, num_groups)
+    dev = x.device
+    q = torch.empty((M, F), dtype=FP8, device=dev) if rowwise else None
+    s = torch.empty((M, F // TILE), dtype=torch.float32, device=dev) if rowwise else None
+    q_t = torch.empty((F, ld_t), dtype=FP8, device=dev)
+    s_t = torch.empty((ld_t // TILE, F), dtype=torch.float32, device=dev)
+    h = torch.empty((M, F), dtype=torch.bfloat16, device=dev) if return_activation else None
+    ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
+    check(
+        lib().aamd_gelu_quant_1x128_dual_grouped(
+            ptr(x), ptr(dh), M, F, F, ptr(group_offsets), num_groups, ptr(ws), ptr(h),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, stream(),
+        )
+    )  # fmt: skip
+    return (q, s, q_t, s_t, h) if return_activation else (q, s, q_t, s_t)
+
+
 def block_quant_batched(w: torch.Tensor, eps: float = 0.0, return_transpose: bool = False):
     """128x128 block quantisation of ``w [E, N, K]`` in one launch.
     Returns ``(q [E,N,K], s [E,N/128,K/128], q_t [E,K,N] | None, s_t [E,K/128,N/128] | None)``."""

@@ -151,6 +151,23 @@ int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void *dh, int64_t ld_dh, cons
                                              int64_t ld_t, void *stream);
 
 /*
+ * GELU, the expert MLP's default activation, fused into the same quantisers:
+ *   h = bf16(x/2 * (1 + erf(x / sqrt 2)))  computed in fp32 from bf16 x, quantised like aamd_quant_1x128 /
+ *   aamd_quant_1x128_dual_grouped would quantise h; with dh != NULL the dual form quantises the gradient
+ *   g = bf16(dh * (cdf(x) + x * pdf(x))) instead (autograd's gelu_backward).
+ * Replaces self.activation = torch.nn.functional.gelu, atorch/modules/moe/grouped_gemm_moe.py:449, applied at
+ * :849 between the gmm calls, and what autograd runs for it, each followed by the per-expert
+ * quantize_op.quantize of the next grouped GEMM's operand (quantized_grouped_linear.py:90-101, 202-206).
+ *   x [rows, F] bf16 (row stride ld), F % 128 == 0; dh [rows, F] bf16 with the same row stride ld
+ *   h_out [rows, F] bf16 or NULL (h, or g in the backward form); other arguments as the SwiGLU forms.
+ */
+int aamd_gelu_quant_1x128(const void *x, int64_t rows, int64_t F, int64_t ld, void *h_out, uint8_t *q, float *s,
+                          void *stream);
+int aamd_gelu_quant_1x128_dual_grouped(const void *x, const void *dh, int64_t M, int64_t F, int64_t ld,
+                                       const int64_t *group_offsets, int E, int32_t *tile_ws, void *h_out, uint8_t *q,
+                                       float *s, uint8_t *q_t, float *s_t, int64_t ld_t, void *stream);
+
+/*
  * Ragged grouped block-scaled GEMM, "NT": for every group g and its rows m,
  *   C[m, n] = sum_kb dot(A[m, kb], B_g[n, kb]) * a_s[m, kb] * b_s_g[n/128 or n, kb]  (+ bias_g[n])
  * fp8 x fp8 MFMA, fp32 accumulation, scales applied per 128-deep block.

@@ -217,6 +217,21 @@ def bias_gather_bgrad(grad: torch.Tensor, bin_ids: torch.Tensor, num_experts: in
     return out
 
 
+def gelu(x: torch.Tensor) -> torch.Tensor:
+    """The expert MLP's default activation, ``torch.nn.functional.gelu`` (grouped_gemm_moe.py:449, applied
+    at :849), on a bf16 tensor: the reference's own op evaluated on the CPU (fp32 inside, one rounding)."""
+    assert x.dtype == torch.bfloat16
+    return torch.nn.functional.gelu(x.detach())
+
+
+def gelu_bwd(dh: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """What autograd runs for that op: ``dh * (cdf(x) + x * pdf(x))`` in fp32, rounded to bf16."""
+    assert x.dtype == torch.bfloat16 and dh.dtype == torch.bfloat16
+    leaf = x.detach().clone().requires_grad_(True)
+    torch.nn.functional.gelu(leaf).backward(dh)
+    return leaf.grad
+
+
 def torch_swiglu(fc1: torch.Tensor) -> torch.Tensor:
     """The reference's own two torch ops (CPU)."""
     a, b = torch.chunk(fc1, 2, dim=-1)

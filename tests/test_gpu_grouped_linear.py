@@ -407,3 +407,78 @@ def test_module_accepts_fp16_activations(dev, oracle):
     for i in range(E):
         g = mod.get_parameter(f"weight{i}").grad
         assert g.dtype == torch.float16 and rel_err(g.float().cpu(), orc["wgrad"][i]) <= TOL
+
+
+@pytest.mark.parametrize("variant", ["swiglu_separate", "swiglu_separate_kn", "gelu", "gelu_bias", "swiglu_bias"])
+def test_grouped_mlp_bodies_match_oracle_composition(oracle, dev, variant):
+    """The other bodies of compute_moe (grouped_gemm_moe.py:836-855): separate gate / up weights (:840-843),
+    GELU (:449, :849) and the use_bias composition with bias_gather_add (:846-853), forward and backward,
+    against the CPU composition: oracle grouped linear (+ bias), the reference's activation op under
+    torch autograd, oracle grouped linear (+ bias).  Tolerances as for the merged SwiGLU body."""
+    from atorch_amd.expert_mlp import grouped_mlp
+
+    E, H, F, M = 3, 256, 384, 416
+    splits = [200, 0, 216]
+    glu = variant.startswith("swiglu")
+    separate = "separate" in variant
+    kn = variant.endswith("_kn")  # first weights stored [E, H, *] (transpose_w1 = False)
+    use_bias = variant.endswith("_bias")
+    n1 = 2 * F if glu else F
+    x = randn_bf16((M, H), 1)
+    w1 = randn_bf16((E, n1, H), 2, std=0.05)  # logical [E, N1, H]: gate rows on top of up rows
+    w2 = randn_bf16((E, F, H), 3, std=0.05)
+    dy = randn_bf16((M, H), 4, std=1e-2)
+    b1 = randn_bf16((E, n1), 5, std=0.5) if use_bias else None
+    b2 = randn_bf16((E, H), 6, std=0.5) if use_bias else None
+
+    def store(w):  # logical [E, n, H] -> the parameter's storage orientation
+        return (w.transpose(1, 2).contiguous() if kn else w.contiguous()).to(dev).requires_grad_(True)
+
+    xg = x.to(dev).requires_grad_(True)
+    w2g = w2.to(dev).requires_grad_(True)
+    if separate:
+        w1g, v1g = store(w1[:, :F]), store(w1[:, F:])
+    else:
+        w1g, v1g = store(w1), None
+    b1g = b1.to(dev).requires_grad_(True) if use_bias else None
+    b2g = b2.to(dev).requires_grad_(True) if use_bias else None
+    out = grouped_mlp(xg, w1g, w2g, torch.tensor(splits), v1=v1g, b1=b1g, b2=b2g,
+                      activation="swiglu" if glu else "gelu", transpose_w1=not kn)  # fmt: skip
+    out.backward(dy.to(dev))
+
+    r1 = oracle.grouped_linear_fwd_bwd(x, [w1[e] for e in range(E)], splits, biases=[b1[e] for e in range(E)] if use_bias else None)
+    fc1 = r1["out"].bfloat16().requires_grad_(True)
+    h = oracle.torch_swiglu(fc1) if glu else torch.nn.functional.gelu(fc1)
+    w2_t = [w2[e].t().contiguous() for e in range(E)]
+    r2 = oracle.grouped_linear_fwd_bwd(h.detach(), w2_t, splits, dy, biases=[b2[e] for e in range(E)] if use_bias else None)
+    h.backward(r2["dgrad"].bfloat16())
+    r1b = oracle.grouped_linear_fwd_bwd(x, [w1[e] for e in range(E)], splits, fc1.grad)
+
+    def close(got, ref):
+        got, ref = got.double(), ref.double()
+        rms = ref.pow(2).mean().sqrt().clamp_min(1e-30)
+        return float((got - ref).pow(2).mean().sqrt() / rms) < 1e-2 and rel_err(got, ref) < 0.15
+
+    assert close(out.detach().cpu().float(), r2["out"])
+    assert close(xg.grad.cpu().float(), r1b["dgrad"])
+
+    def logical(g):  # gradient in storage orientation -> [E, n, H]
+        g = g.cpu().float()
+        return g.transpose(1, 2) if kn else g
+
+    dw1 = torch.cat([logical(w1g.grad), logical(v1g.grad)], dim=1) if separate else logical(w1g.grad)
+    for e in range(E):
+        if splits[e] == 0:
+            continue
+        assert close(dw1[e], r1b["wgrad"][e])
+        assert close(w2g.grad[e].cpu().float(), r2["wgrad"][e].t())
+        if use_bias:
+            assert close(b2g.grad[e].cpu().float(), r2["bgrad"][e])
+            assert close(b1g.grad[e].cpu().float(), r1b["bgrad"][e])
+    assert torch.all(w2g.grad[1] == 0) and torch.all(w1g.grad[1] == 0)
+    if use_bias:
+        assert torch.all(b1g.grad[1] == 0) and torch.all(b2g.grad[1] == 0)
+    with torch.no_grad():
+        out2 = grouped_mlp(x.to(dev), w1g.detach(), w2g.detach(), torch.tensor(splits), v1=v1g.detach() if separate else None,
+                           b1=b1g, b2=b2g, activation="swiglu" if glu else "gelu", transpose_w1=not kn)  # fmt: skip
+    assert torch.equal(out2, out.detach())

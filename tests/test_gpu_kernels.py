@@ -795,3 +795,66 @@ def test_grouped_gemm_random_shapes(dev):
         assert rel_err(dw.cpu(), refw.float().cpu()) <= GEMM_TOL_F32, (case, M, N, K, E)
         # the sum with the old values rounds once more in fp32
         assert rel_err((acc - base).cpu(), refw.float().cpu()) <= 4 * GEMM_TOL_F32, (case, M, N, K, E)
+
+
+# ------------------------------------------------------------------------------------------
+# GELU (the expert MLP's default activation) fused into the quantisers
+# ------------------------------------------------------------------------------------------
+def _gelu_close(got, ref, x):
+    """One bf16 unit in the last place of the result (up to 2^-7 of it) plus a few fp32 roundings of 1 + erf(x / sqrt 2) scaled by |x| (that sum
+    cancels for x << 0, where device and host erf legitimately differ); and, where nothing cancels
+    (x >= -4), at most one unit in the last place on a small fraction of the inputs."""
+    got, ref, x = got.cpu(), ref.cpu(), x.cpu()
+    err = (got.double() - ref.double()).abs()
+    bound = 2.0**-7 * ref.double().abs() + 2.0**-21 * x.double().abs().clamp_min(1.0) + 1e-37
+    assert bool((err <= bound).all()), float((err / bound).max())
+    mid = x.float() >= -4.0
+    d = _ulp_diff(got, ref)
+    d = torch.where(got.float() == ref.float(), torch.zeros_like(d), d)[mid]
+    assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 5e-3
+
+
+def test_gelu_forward_and_backward_over_all_bf16_values(oracle, dev):
+    """h = gelu(x) and g = dh * gelu'(x) from the fused kernels against the oracle (torch's CPU op and its
+    autograd) for every bf16 x of sensible magnitude; codes and scales are exactly the quantisation of
+    the kernel's own values."""
+    from atorch_amd import kernels
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    # beyond 2^100 the op's own fp32 product x (1 + erf) overflows; below 2^-100 the CPU op flushes the
+    # denormal result x / 2 to zero and the device keeps it: neither occurs among activations
+    ax = bits.float().abs()
+    x = bits[(ax < 2.0**100) & ((ax > 2.0**-100) | (ax == 0))]
+    x = x[: x.numel() // 128 * 128].view(-1, 128).contiguous()
+    g = torch.Generator().manual_seed(24)
+    dh = torch.randn(x.shape, generator=g).bfloat16()
+    M = x.shape[0]
+    q, s, h = kernels.gelu_tile_quant(x.to(dev), return_activation=True)
+    _gelu_close(h, oracle.gelu(x), x)
+    qo, so = oracle.tile_quant(h.cpu())
+    assert torch.equal(_u8(q), qo) and torch.equal(s.cpu(), so)
+    goff = kernels.group_offsets_from_splits([M], dev)
+    qb, sb, qb_t, sb_t, gr = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, 1, dh=dh.to(dev), return_activation=True)
+    _gelu_close(gr, oracle.gelu_bwd(dh, x), x)
+    qo, so = oracle.tile_quant(gr.cpu())
+    assert torch.equal(_u8(qb), qo) and torch.equal(sb.cpu(), so)
+
+
+@pytest.mark.parametrize("backward", [False, True], ids=["fwd", "bwd"])
+def test_gelu_quant_dual_grouped(oracle, dev, backward):
+    """The fused kernels equal GELU (or its backward) followed by the dual grouped quantisation: outputs
+    bit-identical to tile_quant_dual_grouped of their own activation / gradient."""
+    from atorch_amd import kernels
+
+    M, F, E = 1000, 384, 5
+    splits = ragged_splits(M, E, seed=25)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    x = randn_bf16((M, F), 26, std=2.0).to(dev)
+    dh = randn_bf16((M, F), 27, std=0.5).to(dev) if backward else None
+    q, s, q_t, s_t, h = kernels.gelu_tile_quant_dual_grouped(x, goff, E, dh=dh, return_activation=True)
+    ref = oracle.gelu_bwd(dh.cpu(), x.cpu()) if backward else oracle.gelu(x.cpu())
+    _gelu_close(h, ref, x)
+    q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(h, goff, E, ld_t=q_t.shape[1])
+    ptot = kernels.padded_total(splits)
+    assert torch.equal(_u8(q), _u8(q2)) and torch.equal(s, s2)
+    assert torch.equal(s_t[: ptot // TILE], s_t2[: ptot // TILE]) and torch.equal(_u8(q_t[:, :ptot]), _u8(q_t2[:, :ptot]))

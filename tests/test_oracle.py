@@ -424,3 +424,37 @@ def test_bias_gather_add_matches_torch(oracle):
         exact = torch.zeros(E, H, dtype=torch.float64).index_add_(0, ids, small.double())
         assert torch.equal(oracle.bias_gather_bgrad(small, ids, E).double(), exact)
 
+
+
+def test_gelu_oracle_against_the_closed_form_over_all_bf16_values(oracle):
+    """oracle.gelu / gelu_bwd (torch's CPU op and its autograd) against x/2 (1 + erf(x/sqrt 2)) and
+    dh (cdf + x pdf) evaluated in float64, for every finite bf16 x.  The op works in fp32, where
+    1 + erf(x/sqrt 2) cancels for x << 0, so the bound is one bf16 rounding of the result plus an fp32
+    rounding of x; where neither cancellation nor denormals play (1e-30 <= |x| <= 4) the results agree
+    to one unit in the last place."""
+    import math
+
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    x = bits[bits.float().abs() < 2.0**100]  # beyond, the op's own fp32 product x (1 + erf) overflows
+    x64 = x.double()
+    cdf = 0.5 * (1.0 + torch.special.erf(x64 / math.sqrt(2.0)))
+    pdf = torch.exp(-0.5 * x64 * x64) / math.sqrt(2.0 * math.pi)
+    g = torch.Generator().manual_seed(3)
+    dh = torch.randn(x.shape, generator=g).bfloat16()
+    mid = (x64.abs() >= 1e-30) & (x64.abs() <= 4.0)
+
+    def ulps(a, b):
+        d = (a.view(torch.int16).int() - b.view(torch.int16).int()).abs()
+        return torch.where(a.float() == b.float(), torch.zeros_like(d), d)
+
+    for got, ref64 in ((oracle.gelu(x), x64 * cdf), (oracle.gelu_bwd(dh, x), dh.double() * (cdf + x64 * pdf))):
+        err = (got.double() - ref64).abs()
+        scale = x64.abs() if got is not None else None
+        bound = 2.0**-8 * ref64.abs() + 2.0**-22 * torch.maximum(scale, torch.ones_like(scale)) + 1e-37
+        assert bool((err <= bound).all()), float((err / bound).max())
+        d = ulps(got, ref64.to(torch.bfloat16))[mid]
+        assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 5e-3
+    # known answers: gelu(0) = 0, gelu(large) = x, gelu(-large) = -0; gelu'(0) = 1/2, gelu'(large) = 1
+    assert oracle.gelu(torch.tensor([0.0, 40.0, -40.0]).bfloat16()).float().tolist() == [0.0, 40.0, -0.0]
+    one = torch.ones(3).bfloat16()
+    assert oracle.gelu_bwd(one, torch.tensor([0.0, 40.0, -40.0]).bfloat16()).float().tolist() == [0.5, 1.0, 0.0]
