@@ -64,6 +64,7 @@ SIGNATURES = {
     "aamd_clock_probe": (_int, [_vp, _i64, _vp]),
     "aamd_stream_probe": (_int, [_vp, _vp, _int, _int, _i64, _i64, _vp]),
     "aamd_mfma_probe": (_int, [_vp, _int, _int, _int, _vp, _vp, _vp]),
+    "aamd_loop_probe": (_int, [_vp, _i64, _int, _int, _vp, _vp, _vp]),
     "aamd_unpermute_combine": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _i64, _int, _vp, _vp]),
     "aamd_permute_rows_scaled": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp, _int, _vp]),
     "aamd_unpermute_probs_grad": (_int, [_vp, _int, _vp, _int, _i64, _i64, _vp, _i64, _int, _vp, _vp]),

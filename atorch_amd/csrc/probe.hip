@@ -79,6 +79,131 @@ __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(const int* __restric
   if (tid == 64 && blockIdx.x == 0) cyc[0] = t1 - t0;  // a wave that shares its SIMD's pipe for the whole run
 }
 
+// Loop model: the instruction sequence of one 128-deep step of the 256 x 256 GEMM configuration on private data -
+// per wave sixteen MFMAs in eight chained pairs, the fold of every pair, the 24 fragment reads of the step from an
+// LDS tile laid out and swizzled like the GEMM's (each fragment is read two pairs before its MFMAs), and eight
+// 1 KB direct-to-LDS loads - without scales, barriers, prologue or epilogue.  With STREAM the loads walk 1 MiB
+// panels of 256 rows of 4 KB (128 bytes per row and step) that the workgroups of an XCD share the way the GEMM's
+// tiles share operand panels (8 + 4 panels for 32 workgroups), moving on to the next set of 96 panels every 32 steps
+// (the buffer holds panel_bytes / 96 MiB sets and wraps); otherwise they re-read 4 KB that stay in the caches.
+// Without SYNC nothing waits for the loads or for other waves: the probe then shows how far the issue of the loads
+// alone holds the MFMAs up.  With SYNC the step has the GEMM's two workgroup barriers (at its start and before the
+// last R row), the second one behind a wait for the loads of the step before, and the loads go out where the GEMM
+// issues them (L slabs behind the first four pairs, R slabs two at a time behind the last two).
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+template <bool STREAM, bool SYNC>
+__global__ __launch_bounds__(512, 1) void loop_probe_kernel(const uint8_t* __restrict__ panels, int n_sets,
+                                                             float* __restrict__ out, int iters, unsigned long long* cyc) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds[128 * 1024];
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  for (int i = tid; i < 128 * 1024 / 16; i += 512) reinterpret_cast<v4i*>(lds)[i] = v4i{0, 0, 0, 0};
+  __syncthreads();
+  const int l32 = lane & 31, hg = lane >> 5, sw = (l32 & 7) ^ ((l32 >> 3) & 1);
+  const int wr = wave & 1, wl = ((wave & 3) >> 1) + 2 * (wave >> 2);
+  uint32_t la[2][2], ra[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const int chk = ((4 * h + 2 * hg + c) ^ sw) << 4;
+      la[h][c] = (uint32_t)(uintptr_t)(lds_ptr_t)lds + (uint32_t)((wl * 64 + l32) * 128 + chk);
+      ra[h][c] = (uint32_t)(uintptr_t)(lds_ptr_t)lds + 65536 + (uint32_t)((wr * 128 + l32) * 128 + chk);
+      asm volatile("" : "+v"(la[h][c]));
+      asm volatile("" : "+v"(ra[h][c]));
+    }
+  typedef const __attribute__((address_space(3))) v4i* lds_v4i_t;
+  auto frag = [&](const uint32_t (&base)[2][2], int sub, int h) {
+    const v4i lo = *(lds_v4i_t)(uintptr_t)(base[h][0] + (uint32_t)(sub * 4096));
+    const v4i hi = *(lds_v4i_t)(uintptr_t)(base[h][1] + (uint32_t)(sub * 4096));
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  // loads: lane l fetches 16 bytes of row l / 8 of an 8-row slab; slab n of this wave starts at row 8 wave + 64 n
+  const uint32_t voff = (uint32_t)(lane >> 3) * 4096u + (uint32_t)((lane & 7) << 4);
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int lp0 = xcd * 8 + (idx & 7), rp0 = 64 + xcd * 4 + ((idx >> 3) & 3);  // panel indices inside a set of 96
+  const uint32_t ldst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds + 98304 + wave * 4096);
+  int kstep = 0;
+  auto dma = [&](int n) {
+    // every 32 steps (one 4 KB row) the workgroups move on to the next set of 96 panels, like tiles to new operands
+    const int set = (kstep >> 5) % n_sets;
+    const uint8_t* g = STREAM ? panels + (size_t)(set * 96 + ((n & 4) ? rp0 : lp0)) * (1u << 20) +
+                                    (size_t)((wave * 8 + 64 * (n & 3)) * 4096) + (kstep & 31) * 128
+                              : panels + (n & 3) * 1024;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(g),
+                 "s"(ldst + (uint32_t)((n & 3) * 1024)) : "memory");
+  };
+  v8i lf[2][2], rf[2][2];
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      lf[j][h] = frag(la, j, h);
+      rf[j][h] = frag(ra, j, h);
+    }
+  v16f acc[2][2], zero, pr;
+#pragma unroll
+  for (int r = 0; r < 16; r++) zero[r] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) acc[i][j] = zero;
+  const float sc = 1.0f + 1e-7f * (float)(tid & 3);
+  const unsigned long long t0 = __builtin_readcyclecounter();
+  for (int it = 0; it < iters; it++) {
+    kstep = it;
+    if (SYNC) {
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+#pragma unroll
+    for (int p = 0; p < 8; p++) {
+      const int i = p >> 1, j = p & 1;
+      __builtin_amdgcn_sched_barrier(0);
+      pr = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i & 1][0], lf[j][0], zero, 0, 0, 0, 0, 0, 0);
+      pr = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i & 1][1], lf[j][1], pr, 0, 0, 0, 0, 0, 0);
+      asm volatile("" : "+v"(pr));
+      __builtin_amdgcn_sched_barrier(0);
+      if (!SYNC || p < 4) dma(p);
+      if (j == 0 && i + 1 < 4) {  // the next R row while this one is in use
+        rf[(i + 1) & 1][0] = frag(ra, i + 1, 0);
+        rf[(i + 1) & 1][1] = frag(ra, i + 1, 1);
+      }
+      if (p == 5) {  // first R row of the next step
+        if (SYNC) {  // all but this step's four L slabs have landed
+          __builtin_amdgcn_sched_barrier(0);
+          asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        rf[0][0] = frag(ra, 0, 0);
+        rf[0][1] = frag(ra, 0, 1);
+      }
+      if (p >= 6) {  // L fragments of the next step
+        if (SYNC) {
+          dma(4 + (p - 6) * 2);
+          dma(5 + (p - 6) * 2);
+        }
+        lf[p - 6][0] = frag(la, p - 6, 0);
+        lf[p - 6][1] = frag(la, p - 6, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i & 1][j][r] = __builtin_fmaf(pr[r], sc, acc[i & 1][j][r]);
+      asm volatile("" : "+v"(acc[i & 1][j]));
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  const unsigned long long t1 = __builtin_readcyclecounter();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) s += acc[i][j][r];
+  out[(size_t)blockIdx.x * 512 + tid] = s;
+  if (tid == 64 && blockIdx.x == 0) cyc[0] = t1 - t0;
+}
+
 // Streaming probe: what this GPU's memory system delivers for a given mix of read and write streams with
 // nothing else in the way.  Every lane handles 16-byte words: per unit of work it reads one word from
 // each of R input streams and writes one word to each of W output streams (streams are disjoint
@@ -159,6 +284,23 @@ extern "C" int aamd_clock_probe(uint64_t* out, int64_t min_cycles, void* stream)
   AAMD_REQUIRE(min_cycles >= 0 && min_cycles <= (1LL << 31), "clock_probe: min_cycles out of range");
   aamd::clock_probe_kernel<<<1, 64, 0, (hipStream_t)stream>>>(reinterpret_cast<unsigned long long*>(out), min_cycles);
   AAMD_LAUNCH_CHECK("clock_probe");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_loop_probe(const void* panels, int64_t panel_bytes, int stream_panels, int iters, float* out,
+                               uint64_t* cycles, void* stream) {
+  AAMD_REQUIRE(panels && out && cycles, "loop_probe: null pointer");
+  AAMD_REQUIRE(iters >= 1 && iters <= (1 << 20), "loop_probe: bad iteration count");
+  AAMD_REQUIRE(panel_bytes >= (stream_panels ? (int64_t)96 << 20 : (int64_t)4096),
+               "loop_probe: the panel buffer holds 96 MiB (64 + 32 panels of 1 MiB) when the loads stream, 4 KB otherwise");
+  AAMD_REQUIRE((reinterpret_cast<uintptr_t>(panels) & 15) == 0, "loop_probe: panels must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int n_sets = (int)(panel_bytes / ((int64_t)96 << 20));
+  unsigned long long* cy = (unsigned long long*)cycles;
+  if (stream_panels == 2) aamd::loop_probe_kernel<true, true><<<256, 512, 0, st>>>((const uint8_t*)panels, n_sets, out, iters, cy);
+  else if (stream_panels) aamd::loop_probe_kernel<true, false><<<256, 512, 0, st>>>((const uint8_t*)panels, n_sets, out, iters, cy);
+  else aamd::loop_probe_kernel<false, false><<<256, 512, 0, st>>>((const uint8_t*)panels, 1, out, iters, cy);
+  AAMD_LAUNCH_CHECK("loop_probe");
   return AAMD_OK;
 }
 

@@ -45,7 +45,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "quant"],
+                    help="c1-c5: the configurations of the benchmark; quant: every quantisation kernel of the path at "
+                         "the c2 shapes, each beside the streaming probe of its read:write mix")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--operands", default="random", choices=["random", "zeros"],
                     help="GEMM workloads: 'zeros' clears the fp8 codes of the activations and weights after set-up; "
@@ -160,6 +162,36 @@ def mfma_probe(kernels, dev, iters=3000):
                 # with the fold the two waves of a SIMD alternate on its pipe, so the probed wave runs for the
                 # whole of its round (one of wgs/256): its cycle count over that time is the shader clock
                 res[key]["sclk_ghz"] = round(int(cyc.item()) / (ms * 1e6 / (wgs / 256)), 3)
+    return res
+
+
+def loop_probe(dev, iters=2000):
+    """One step of the 256 x 256 GEMM loop as an instruction sequence on private data (zero codes): shader
+    cycles per step as one wave sees them (2048 of them are MFMA work) and TFLOP/s by the clock, with
+    cache-resident loads, with loads that stream shared panels, and with the GEMM's barriers and waits."""
+    from atorch_amd._lib import check, lib
+
+    panels = torch.zeros(16 * (96 << 20), dtype=torch.uint8, device=dev)  # 1.5 GiB: more than the last-level cache
+    out = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    cyc = torch.zeros(1, dtype=torch.int64, device=dev)
+    res = {}
+    for name, stream_panels, nbytes in (("resident_loads", 0, 96 << 20), ("streaming_panels_96MiB", 1, 96 << 20),
+                                        ("streaming_panels_1.5GiB", 1, panels.numel()),
+                                        ("streaming_panels_1.5GiB_barriers_and_waits", 2, panels.numel())):
+        st = torch.cuda.current_stream().cuda_stream
+        call = lambda: check(lib().aamd_loop_probe(panels.data_ptr(), nbytes, stream_panels, iters,  # noqa: E731
+                                                   out.data_ptr(), cyc.data_ptr(), st))
+        call()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        call()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b)
+        c = int(cyc.item()) / iters
+        res[name] = {"cycles_per_step": round(c, 1), "mfma_share_of_cycles": round(2048.0 / c, 4),
+                     "TFLOP/s": round(256 * 8 * iters * 16 * 131072.0 / ms / 1e9, 1)}  # fmt: skip
     return res
 
 
@@ -360,6 +392,9 @@ def run_gemm(args, kernels, dev):
                                   "achieved_tflops": round(wg_flops / (wg_avg * 1e-3) / 1e12, 2),
                                   "frac": round(wg_flops / (wg_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
 
+    if args.workload == "c2" and not args.no_extras and args.operands == "random":
+        extras["forward_gemm_by_operand_data"] = operand_data_probe(kernels, layers[0], dev)
+
     cpu = None
     if not args.no_cpu_baseline and args.operands == "random":
         cpu = cpu_gemm_baseline(layers[0], counts)
@@ -375,6 +410,31 @@ def run_gemm(args, kernels, dev):
         "cpu_baseline": cpu,
         "extras": extras,
     }  # fmt: skip
+
+
+def operand_data_probe(kernels, layer, dev, iters=5):
+    """The first layer's forward launch with its own codes and with all-zero codes (same scales, sizes and
+    addresses pattern): the instruction stream is the same, what differs is the switching activity of the
+    matrix pipes, which the GPU's power management answers with the shader clock."""
+    res = {}
+    zx, zw = torch.zeros_like(layer.qx.view(torch.uint8)), torch.zeros_like(layer.qw.view(torch.uint8))
+    out = torch.empty_like(layer.y)  # the layer's own output stays as the timed steps left it
+    for name, qx, qw in (("benchmark_codes", layer.qx, layer.qw), ("zero_codes", zx.view(layer.qx.dtype), zw.view(layer.qw.dtype))):
+        fn = lambda: kernels.grouped_gemm_nt(qx, layer.sx, qw, layer.sw, layer.goff, out=out)  # noqa: E731
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / iters
+        tf = layer.flops / ms / 1e9
+        res[name] = {"TFLOP/s": round(tf, 1), "frac": round(tf / PEAK_FP8_TFLOPS, 4), "avg_launch_ms": round(ms, 4),
+                     "sclk_ghz": clock_under(fn, dev)}  # fmt: skip
+    del zx, zw, out
+    return res
 
 
 def cpu_gemm_baseline(layer, counts):
@@ -463,6 +523,14 @@ def run_c5(args, kernels, dev):
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_quant_baseline(x, idx)
+    mixes = None
+    if args.workload == "c5" and not args.no_extras:
+        # what plain streaming kernels reach with each kernel's ratio of bytes read to bytes written
+        del y
+        torch.cuda.empty_cache()
+        pr = mix_probe(dev, ["1:4", "8:1", "2:1"])
+        mixes = {"permute_quant (1:4)": pr["1:4"]["GB/s"], "unpermute_combine (8:1)": pr["8:1"]["GB/s"],
+                 "tile_quant_plain (2:1)": pr["2:1"]["GB/s"]}  # fmt: skip
     return {
         "metric": "quant/permute HBM GB/s (permute+1x128 quant and unpermute+combine)",
         "value": round(total_gbs, 1),
@@ -483,6 +551,7 @@ def run_c5(args, kernels, dev):
             "tile_quant_plain": {"GB/s": round(tq, 1), "frac": round(tq / PEAK_HBM_GBS, 4),
                                  "avg_launch_ms": round(tq_ms, 4), "bytes_per_launch": tq_bytes},
             "moe_preprocess_ms": round(pre_ms, 4),
+            "mix_probe_GB/s": mixes,
         },
     }  # fmt: skip
 
@@ -509,6 +578,68 @@ def cpu_quant_baseline(x, idx):
                       f"cast ({dt:.2f} s)"}  # fmt: skip
 
 
+# ------------------------------------------------------------------------------------------
+# quant: the quantisation kernels of the expert MLP at the c2 shapes
+# ------------------------------------------------------------------------------------------
+def run_quant(args, kernels, dev):
+    E, T, k, F = 8, 16384, 2, 14336
+    idx, _ = routing(T, E, k, dev)
+    _, _, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
+    M = T * k
+    q1 = 1 + 4 / TILE  # bytes written per element by one 1x128 quantisation (code + its share of the scale)
+    x = randn((M, F), dev, 1.0, 1)
+    fc1 = randn((M, 2 * F), dev, 1.0, 2)
+    dh = randn((M, F), dev, 1e-2, 3)
+    w = randn((E, 2 * F, 4096), dev, 0.02, 4)
+    # name: (call, algorithmic bytes, read:write mix of the streaming probe in equal-sized streams)
+    cases = {
+        "quant_1x128": (lambda: kernels.tile_quant(x), M * F * (2 + q1), "2:1"),
+        "quant_1x128_dual_grouped": (lambda: kernels.tile_quant_dual_grouped(x, goff, E), M * F * (2 + 2 * q1), "1:1"),
+        "swiglu_quant_1x128": (lambda: kernels.swiglu_tile_quant(fc1), M * F * (4 + q1), "4:1"),
+        "swiglu_quant_1x128_dual_grouped": (lambda: kernels.swiglu_tile_quant_dual_grouped(fc1, goff, E),
+                                            M * F * (4 + 2 * q1), "2:1"),
+        "swiglu_bwd_quant_1x128_dual_grouped": (lambda: kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E),
+                                                M * F * (6 + 4 * q1), "3:2"),
+        "quant_128x128": (lambda: kernels.block_quant_batched(w), w.numel() * 3, "2:1"),
+        "quant_128x128_with_transpose": (lambda: kernels.block_quant_batched(w, return_transpose=True),
+                                         w.numel() * 4, "1:1"),
+    }  # fmt: skip
+    res, tot_b, tot_ms = {}, 0.0, 0.0
+    for name, (fn, nbytes, mix) in cases.items():
+        for _ in range(max(args.warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(args.steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / args.steps
+        gbs = nbytes / ms / 1e6
+        res[name] = {"GB/s": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4), "avg_launch_ms": round(ms, 4),
+                     "bytes_per_launch": int(nbytes), "mix": mix}  # fmt: skip
+        tot_b += nbytes
+        tot_ms += ms
+    del x, fc1, dh, w
+    torch.cuda.empty_cache()
+    probe = mix_probe(dev, sorted({v[2] for v in cases.values()}))
+    for name, (_, _, mix) in cases.items():
+        res[name]["mix_probe_GB/s"] = probe[mix]["GB/s"]
+        res[name]["frac_of_mix_probe"] = round(res[name]["GB/s"] / probe[mix]["GB/s"], 4)
+    worst = min(res, key=lambda n: res[n]["frac"])
+    total = tot_b / tot_ms / 1e6
+    return {
+        "metric": "quantisation kernels HBM GB/s (c2 shapes, all kernels one after the other)",
+        "value": round(total, 1), "unit": "GB/s", "ms_per_step": round(tot_ms, 4), "dtype": "fp8",
+        "config": {"workload": "quant: 32768 routed rows of 14336 features in 8 groups, weights 8 x 28672 x 4096, bf16 in"},
+        "roofline": {"kernel": worst, "bound": "hbm", "achieved": res[worst]["GB/s"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": res[worst]["frac"], "traffic": None},
+        "cpu_baseline": None,
+        "extras": {"kernels": res},
+    }  # fmt: skip
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -528,7 +659,10 @@ def main():
         print(json.dumps({"metric": "streaming probe GB/s by read:write mix", "unit": "GB/s", "n_gpus": 1,
                           "mixes": mix_probe(dev, mixes)}))  # fmt: skip
         return
-    res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
+    if args.workload == "quant":
+        res = run_quant(args, kernels, dev)
+    else:
+        res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
     if args.workload == "c2" and not args.no_extras:
         # the other half of the metric (quant / permute GB/s) and the two probes ride along in extras
         torch.cuda.empty_cache()
@@ -543,6 +677,7 @@ def main():
         }  # fmt: skip
         torch.cuda.empty_cache()
         res["extras"]["mfma_probe"] = mfma_probe(kernels, dev)
+        res["extras"]["loop_probe"] = loop_probe(dev)
     out = {
         "metric": res["metric"],
         "value": res["value"],

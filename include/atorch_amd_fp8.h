@@ -313,6 +313,22 @@ int aamd_mfma_probe(const void *operands, int fold, int iters, int workgroups, f
                     void *stream);
 
 /*
+ * Loop probe (no counterpart in the reference; the benchmark reports what one 128-deep step of the
+ * 256 x 256 GEMM configuration costs as an instruction sequence on private data): 256 workgroups of
+ * eight waves run, `iters` times, the step's sixteen MFMAs with their folds, its 24 fragment reads
+ * from an LDS tile laid out like the GEMM's and its eight 1 KB direct-to-LDS loads, without scales,
+ * barriers, prologue or epilogue.  stream_panels == 0: the loads re-read the first 4 KB of `panels`;
+ * != 0: they walk 1 MiB panels (256 rows of 4 KB, 128 bytes per row and step) shared among the
+ * workgroups of an XCD the way the GEMM's tiles share operand panels, and move on to the next set of
+ * 96 panels every 32 steps (`panels` then holds a multiple of 96 MiB: panel_bytes / 96 MiB sets, wrapped);
+ * 2: the same with the GEMM's two barriers per step, the wait for the loads of the step before in front
+ * of the second one, and the loads issued where the GEMM issues them.
+ * FLOP = 256 * 8 * iters * 16 * 131072; out: 256 * 512 floats; cycles[0]: shader cycles of one wave.
+ */
+int aamd_loop_probe(const void *panels, int64_t panel_bytes, int stream_panels, int iters, float *out,
+                    uint64_t *cycles, void *stream);
+
+/*
  * Streaming probe (no counterpart in the reference; the benchmark prices the memory-bound kernels
  * against what the memory system delivers for their mix of read and written bytes): per 16-byte word
  * of work one word is read from each of `reads` input streams and one written to each of `writes`
