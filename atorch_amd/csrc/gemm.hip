@@ -367,7 +367,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // are fetched every eighth step, 16 bytes per thread, into [row][8] floats.  The last batch is
   // shifted back so that it ends at the last block.
   const bool batch = MODE == kRaggedRows && p.ls_batch != 0;  // uniform; implies nkb >= 8
-  const bool step_scale = !(batch && l_side);                 // this wave loads a scale every step
+  // this wave loads a scale every step (never in the configuration that takes all its scales in batches)
+  const bool step_scale = !C::LAHEAD && !(batch && l_side);
   const int brow = (tid >> 1) < lvalid ? (tid >> 1) : lvalid - 1;
   const uint32_t boff = ((uint32_t)brow * (uint32_t)p.ls_row_stride + (uint32_t)(tid & 1) * 4u) * 4u;
   auto batch_start = [&](int b) { return 8 * b + 8 <= nkb ? 8 * b : nkb - 8; };
@@ -405,8 +406,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
                  : "memory");
   };
   auto dmaR_scales = [&](int kb, float* Sd) {
-    if (!l_side) dma_scale(kb, Sd);
-    if (batch && (kb & 7) == 0) dma_scale_batch(kb >> 3);  // lands a step before its first use
+    if constexpr (!C::LAHEAD) {
+      if (!l_side) dma_scale(kb, Sd);
+      if (batch && (kb & 7) == 0) dma_scale_batch(kb >> 3);  // lands a step before its first use
+    }
   };
   auto dmaL_one = [&](int n, int kb, uint8_t* Ld, float* Sd) {
     dmaL_tile(n, kb, Ld);
@@ -634,7 +637,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     // has just issued its MFMAs, and the one that waited folds while those still run.
     // Loads complete in issue order, so "all but the newest L group" is one wait count.  Past the
     // end the loads re-read the last block to keep the counts uniform.
-    static_assert(!R_PER_ROW, "the two-barrier pipeline is written for block-scaled R operands");
+    static_assert(!R_PER_ROW && MODE == kRaggedRows, "the two-barrier pipeline is written for block-scaled R operands");
     static_assert(C::PRB == 1 && C::WTR % 2 == 0 && C::RCH % C::WTL == 0 && C::LCH <= NTILES, "pipeline shape");
     constexpr int PT = (C::WTR - 1) * C::WTL - 1;  // the sub-tile in front of barrier P
     constexpr int RPER = C::RCH / C::WTL;
@@ -646,19 +649,36 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       const v4i hi = *(lds_v4i_t)(uintptr_t)(base[h][1] + delta);
       return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
+    // Scales of this pipeline come in batches of eight contraction blocks only (the launcher takes the other
+    // configuration when K has fewer than eight blocks or the scale rows are not 16-byte aligned), so a
+    // step issues no scale load and takes no branch: batch b (blocks 8 b .. 8 b + 7, the last one shifted
+    // back to end at the last block) is requested behind barrier P of step 8 (b - 1), eight steps before
+    // its first use.  L scales: every wave fetches 32 rows x 32 bytes into LsB[b & 1][row][8]; R block
+    // scales: wave 0 fetches the tile's two 128-row blocks x 32 bytes into RsB[b & 1][block][8] (lanes past
+    // the fourth repeat those addresses: the direct-to-LDS load always writes 1 KB).
+    float* const RsB0 = Sc0;  // [2][NT] floats, the first 16 of each in use
+    const int rblocks = rvalid / kTile;
+    const int rlane_blk = ((lane >> 1) & 1) < rblocks ? (lane >> 1) & 1 : rblocks - 1;
+    const uint32_t roff = ((uint32_t)rlane_blk * (uint32_t)p.rs_row_stride + (uint32_t)(lane & 1) * 4u) * 4u;
+    auto dma_batches = [&](int b) {
+      dma_scale_batch(b);
+      if (wave == 0) {
+        const uint8_t* sb = reinterpret_cast<const uint8_t*>(Rsg + uniform_i64((r0 / kTile) * p.rs_row_stride + batch_start(b)));
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     ::"v"(roff), "s"(sb), "s"(lds_addr(RsB0 + (b & 1) * NT)) : "memory");
+      }
+    };
     if (nkb > 0) {
-      dmaL(0, Lbuf0, Sc0);
+      dmaL(0, Lbuf0, Sc0);  // (the per-step scale hooks of these helpers are off: see step_scale)
       dmaR(0, Rbuf0, Sc0);
+      dma_batches(0);
       dmaL(kclamp(1), Lbuf1, Sc1);
       dmaR(kclamp(1), Rbuf1, Sc1);
-      // the tiles of step 0 have landed; those of step 1 may still be on their way
-      if (step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + C::RCH + kScaleLd) : "memory");
-      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + C::RCH) : "memory");
+      // the tiles of step 0 and the first scale batch have landed; those of step 1 may still be on their way
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + C::RCH) : "memory");
       auto barrier_q = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-      auto barrier_p = [&]() {
-        if (l_side && step_scale) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH + kScaleLd) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory");
-      };
+      // all but this step's L tile loads have landed (loads complete in issue order)
+      auto barrier_p = [&]() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(C::LCH) : "memory"); };
       if (has_work) {
         v8i lf[C::WTL][2], rf[2][2];
         float cs[C::WTL], csn[C::WTL], rblkn;
@@ -666,16 +686,14 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
         v16f pr, zero;
 #pragma unroll
         for (int r = 0; r < 16; r++) zero[r] = pr[r] = 0.f;
-        // scales of step kb, which sit in stage buffer `stage`: the lane's L row scales and the R block
-        // scale of the wave; their product is formed where it is first needed, not where the reads are issued
-        auto read_scales = [&](int kb, int stage, float (&dst)[C::WTL], float& rblk) {
-          const float* Sct = stage ? Sc1 : Sc0;
-          const int bsel = kb >> 3;
-          const float* Lsc = batch ? LsB0 + (bsel & 1) * (BM * 8) + (kb - batch_start(bsel)) : Sct;
-          const int lsc_stride = batch ? 8 : 1;
-          rblk = Sct[BM + wrow0 / kTile];
+        // scales of step kb: the lane's L row scales and the R block scale of the wave; their product is
+        // formed where it is first needed, not where the reads are issued
+        auto read_scales = [&](int kb, float (&dst)[C::WTL], float& rblk) {
+          const int b = kb >> 3, in_batch = kb - batch_start(b);
+          const float* Lsc = LsB0 + (b & 1) * (BM * 8) + in_batch;
+          rblk = RsB0[(b & 1) * NT + (wrow0 / kTile) * 8 + in_batch];
 #pragma unroll
-          for (int j = 0; j < C::WTL; j++) dst[j] = Lsc[(wlrow0 + j * 32 + l32) * lsc_stride];
+          for (int j = 0; j < C::WTL; j++) dst[j] = Lsc[(wlrow0 + j * 32 + l32) * 8];
         };
         // (the empty volatile statements pin MFMAs and folds between the memory instructions around
         // them: plain arithmetic is otherwise free to drift past inline assembly)
@@ -694,19 +712,19 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
         for (int j = 1; j < C::WTL; j++)
 #pragma unroll
           for (int h = 0; h < 2; h++) lf[j][h] = frag(la, 0, BM, j, h);
-        read_scales(0, 0, cs, rblkn);
+        read_scales(0, cs, rblkn);
 #pragma unroll
         for (int j = 0; j < C::WTL; j++) cs[j] *= rblkn;
-        auto step = [&](int kb, auto S) {
+        // FIRST: the first step of a run of eight, which requests the next scale batch behind barrier P
+        auto step = [&](int kb, auto S, auto FIRST) {
           constexpr int s = decltype(S)::value;
+          constexpr bool kFirst = decltype(FIRST)::value;
           uint8_t* const Lc = s ? Lbuf1 : Lbuf0;
           uint8_t* const Rc = s ? Rbuf1 : Rbuf0;
-          float* const Scur = s ? Sc1 : Sc0;
           const int k2 = kclamp(kb + 2);
           __builtin_amdgcn_sched_barrier(0);
           barrier_q();
           __builtin_amdgcn_sched_barrier(0);
-          dmaL_scales(k2, Scur);
           fold(C::WTR - 1, C::WTL - 1, cs_last);  // owed by the step before (adds zero in the first step)
           static_for<NTILES>([&](auto T) {
             constexpr int t = decltype(T)::value;
@@ -726,11 +744,13 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
               __builtin_amdgcn_sched_barrier(0);
               barrier_p();
               __builtin_amdgcn_sched_barrier(0);
-              dmaR_scales(k2, Scur);
+              if constexpr (kFirst) {
+                if (kb + 8 < nkb) dma_batches((kb >> 3) + 1);
+              }
               // row C::WTR - 2 has been consumed: its registers take the first R row of the next step
 #pragma unroll
               for (int h = 0; h < 2; h++) rf[0][h] = frag(ra, s ^ 1, BN, 0, h);
-              read_scales(kclamp(kb + 1), s ^ 1, csn, rblkn);
+              read_scales(kclamp(kb + 1), csn, rblkn);
             }
             if constexpr (t > PT) {
               constexpr int jn = t - PT - 1;  // == j: this sub-tile was the last user of lf[j]
@@ -745,29 +765,37 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #pragma unroll
           for (int j = 0; j < C::WTL; j++) cs[j] = csn[j] * rblkn;
         };
-        int kb = 0;
-        for (; kb + 1 < nkb; kb += 2) {  // two steps per trip: the stage addresses are compile-time constants
-          step(kb, std::integral_constant<int, 0>{});
-          step(kb + 1, std::integral_constant<int, 1>{});
+        // runs of eight steps (the contraction has a multiple of four blocks, at least eight), two steps per
+        // trip so that the stage addresses are compile-time constants
+        constexpr std::integral_constant<int, 0> S0{};
+        constexpr std::integral_constant<int, 1> S1{};
+        for (int kb = 0; kb < nkb; kb += 8) {
+          const int n = nkb - kb < 8 ? nkb - kb : 8;
+          step(kb, S0, std::true_type{});
+          step(kb + 1, S1, std::false_type{});
+          for (int kk = 2; kk < n; kk += 2) {
+            step(kb + kk, S0, std::false_type{});
+            step(kb + kk + 1, S1, std::false_type{});
+          }
         }
-        if (kb < nkb) step(kb, std::integral_constant<int, 0>{});
         __builtin_amdgcn_sched_barrier(0);
         fold(C::WTR - 1, C::WTL - 1, cs_last);
       } else {
-        // a wave without valid rows: loads and barriers only
-        auto step = [&](int kb, uint8_t* Lc, uint8_t* Rc, float* Scur) {
+        // a wave without valid rows: loads and barriers only, in the order of the working waves
+        auto step = [&](int kb, uint8_t* Lc, uint8_t* Rc, bool first) {
           const int k2 = kclamp(kb + 2);
           barrier_q();
-          dmaL(k2, Lc, Scur);
+#pragma unroll
+          for (int n = 0; n < C::LCH; n++) dmaL_tile(n, k2, Lc);
           barrier_p();
-          dmaR(k2, Rc, Scur);
+          if (first && kb + 8 < nkb) dma_batches((kb >> 3) + 1);
+#pragma unroll
+          for (int n = 0; n < C::RCH; n++) dmaR_tile(n, k2, Rc);
         };
-        int kb = 0;
-        for (; kb + 1 < nkb; kb += 2) {
-          step(kb, Lbuf0, Rbuf0, Sc0);
-          step(kb + 1, Lbuf1, Rbuf1, Sc1);
+        for (int kb = 0; kb < nkb; kb += 2) {
+          step(kb, Lbuf0, Rbuf0, (kb & 7) == 0);
+          step(kb + 1, Lbuf1, Rbuf1, false);
         }
-        if (kb < nkb) step(kb, Lbuf0, Rbuf0, Sc0);
       }
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
     }
@@ -988,8 +1016,12 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   AAMD_REQUIRE(K > 0, "grouped_gemm_nt: K must be positive");
   AAMD_REQUIRE(lda < (1LL << 23) && K < (1LL << 23), "grouped_gemm_nt: row stride too large");
   hipStream_t st = (hipStream_t)stream;
-  // tile-scaled B carries per-row R scales: use the configuration that has room for them
-  const bool large = use_large_tiles(((M + 255) / 256 + (group_offsets ? E : 0)) * ((N + 255) / 256), true);
+  // 16-byte loads of scale batches need aligned rows and whole groups of four blocks
+  const bool batches = (K / kBK) >= 8 && (K / kBK) % 4 == 0 && aligned16(a_s) && g_opt.ls_batch != 0;
+  // tile-scaled B carries per-row R scales: use the configuration that has room for them; the 256x256
+  // configuration takes all its scales in batches
+  const bool large = use_large_tiles(((M + 255) / 256 + (group_offsets ? E : 0)) * ((N + 255) / 256), true) &&
+                     (b_tile_scaled || (batches && aligned16(b_s)));
   const int BM = large ? CfgLarge::BM : CfgSmall::BM;
   const int BN = large ? (b_tile_scaled ? CfgWgrad::BN : CfgLarge::BN) : CfgSmall::BN;
   if (group_offsets) {
@@ -998,9 +1030,7 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   }
   GemmParams p = {};
   p.L = a; p.ldl = lda; p.Ls = a_s; p.ls_row_stride = K / kBK; p.ls_blk_stride = 1;
-  // 16-byte loads of scale batches need aligned rows and whole groups of four blocks
-  p.ls_batch = (K / kBK) >= 8 && (K / kBK) % 4 == 0 && (reinterpret_cast<uintptr_t>(a_s) & 15) == 0;
-  if (g_opt.ls_batch == 0) p.ls_batch = 0;
+  p.ls_batch = batches;
   p.R = b; p.ldr = K; p.r_group_stride = N * K;
   p.Rs = b_s;
   p.rs_row_stride = K / kBK; p.rs_blk_stride = 1;
