@@ -79,7 +79,7 @@ struct F16 {
   typedef u16 elem;
 };
 // Inputs whose values are bf16 numbers: quotients by the scale of a bf16 maximum may take the
-// checked three-instruction division (see Divider); fp32 and fp16 inputs take the plain one.
+// checked two-instruction division (see Divider); fp32 and fp16 inputs take the plain one.
 template <typename IN>
 constexpr bool kBf16Values = !std::is_same<IN, F32>::value && !std::is_same<IN, F16>::value;
 
@@ -93,22 +93,21 @@ __device__ __forceinline__ void unpack8(const v4i& raw, float* v) {
 }
 
 // ---- 16-lane (one DPP row) max reduction: every lane of the row gets the max
+// Maximum over the 16 lanes of a DPP row of values that are not negative: such floats order like their bit
+// patterns, and the integer maximum takes its second operand straight from the neighbouring lane (the float
+// one would first canonicalise it).  A NaN orders above every number and is kept.
 template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+  return o > v ? o : v;
 }
 __device__ __forceinline__ float row16_max(float v) {
-  v = fmaxf(v, dpp_f32<0xB1>(v));   // quad_perm [1,0,3,2]
-  v = fmaxf(v, dpp_f32<0x4E>(v));   // quad_perm [2,3,0,1]
-  v = fmaxf(v, dpp_f32<0x141>(v));  // row_half_mirror
-  v = fmaxf(v, dpp_f32<0x140>(v));  // row_mirror
-  return v;
-}
-
-// s = max(amax, eps) / 448 ; 0 -> 1.  IEEE division: the scale is part of the bit-exact contract.
-__device__ __forceinline__ float scale_from_amax(float amax, float eps) {
-  float s = fmaxf(amax, eps) / kFp8Max;
-  return s == 0.f ? 1.f : s;
+  uint32_t u = __float_as_uint(v);
+  u = dpp_max_u32<0xB1>(u);   // quad_perm [1,0,3,2]
+  u = dpp_max_u32<0x4E>(u);   // quad_perm [2,3,0,1]
+  u = dpp_max_u32<0x141>(u);  // row_half_mirror
+  u = dpp_max_u32<0x140>(u);  // row_mirror
+  return __uint_as_float(u);
 }
 
 // Two floats -> two e4m3fn codes in the low or high half of `old` (RNE, v_cvt_pk_fp8_f32).
@@ -120,57 +119,73 @@ __device__ __forceinline__ int pack2_fp8(float a, float b, int old) {
   return __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, HI);
 }
 
-// Division of many values by one scale, correctly rounded like the IEEE division the contract
-// asks for, at three instructions per value: with y the reciprocal of s refined by one Newton
-// step, q = x*y, r = x - s*q (exact in an FMA), q + r*y is the correctly rounded quotient
-// (Markstein's scheme, the tail of the hardware's own division sequence without its per-value
-// range scaling).  Scales whose reciprocal could leave the normal range take the plain division.
-// The scheme is used where it has been checked against the plain division over its whole domain:
-// bf16 values divided by the scale of a bf16 maximum (amax / 448).  fp32 inputs and scales that
-// come from an eps clamp take the plain division.
+// The scale of a tile, s = max(amax, eps) / 448 with 0 -> 1, and what divides the tile's values by it.
+// Scale and quotients are part of the bit-exact contract: they are the correctly rounded (IEEE) ones.
+//
+// `plain` takes the hardware's division sequences, a dozen instructions per quotient.  Without it (amax and
+// the values are bf16 numbers, eps is zero):
+//   scale: the tail of the division sequence with the constant's reciprocal, y = RN(1 / 448): q = a y,
+//     r = a - 448 q (exact in an FMA), s = q + r y (Markstein); checked against a / 448 for every bf16 a.
+//   quotients, two instructions per value: the reciprocal of s is held as an unevaluated sum yh + yl.  yh
+//     lies two units in the last place below the hardware reciprocal, so below 1 / s, and with
+//     e = 1 - s yh > 0 (one FMA), yl = yh (e + e^2) >= +0 makes yh + yl = 1 / s to about 2^-60.  Then
+//     fma(x, yh, x yl) rounds x (yh + yl) once (the small product carries a relative error of 2^-24 on a
+//     term 2^-21 of the sum), and both products of a zero x have its sign, so a negative zero stays one.
+//     That is no proof of a correctly rounded quotient: the scheme is used where every case has been
+//     enumerated and gives the code of the plain division: all pairs of a bf16 value and a bf16 maximum,
+//     about 10^9.
+// Maxima outside 2^-90 .. 2^100 (zero aside) take the plain path, where a residual or a reciprocal could
+// leave the normal range.
 struct Divider {
-  float s, y;
+  float s, yh, yl;
   bool plain;
 };
-__device__ __forceinline__ Divider make_divider(float s, bool force_plain) {
+__device__ __forceinline__ Divider make_scale(float amax, float eps, bool plain) {
+  const float a = fmaxf(amax, eps);
   Divider d;
-  d.s = s;
-  const float y0 = __builtin_amdgcn_rcpf(s);
-  const float e = __builtin_fmaf(-s, y0, 1.0f);
-  d.y = __builtin_fmaf(e, y0, y0);
-  d.plain = force_plain || !(s > 0x1p-100f && s < 0x1p100f);
+  d.plain = plain || !(a < 0x1p100f) || (a < 0x1p-90f && a > 0.f);
+  if (__builtin_expect(d.plain, 0)) {
+    const float s = a / kFp8Max;
+    d.s = s == 0.f ? 1.f : s;
+    d.yh = d.yl = 0.f;
+  } else {
+    constexpr float y = 1.0f / kFp8Max;
+    const float q = a * y;
+    const float r = __builtin_fmaf(-kFp8Max, q, a);
+    const float s = __builtin_fmaf(r, y, q);
+    d.s = s == 0.f ? 1.f : s;
+    d.yh = __uint_as_float(__float_as_uint(__builtin_amdgcn_rcpf(d.s)) - 2u);
+    const float e = __builtin_fmaf(-d.s, d.yh, 1.0f);
+    d.yl = __builtin_fmaf(e, e, e) * d.yh;
+  }
   return d;
 }
-__device__ __forceinline__ float neg_div_by(float x, const Divider& d) {
-  const float q = x * d.y;
-  const float r = __builtin_fmaf(-d.s, q, x);
-  // -(q + r*y) as (r)(-y) + (-q): the same rounding, and a zero keeps the (flipped) sign of x: r is
-  // +0 then, so the sum is (-0) + (-q).  The caller flips the sign bits of the packed codes.
-  return __builtin_fmaf(r, -d.y, -q);
+// the divider of a scale that make_scale produced elsewhere (`plain` as it was given there)
+__device__ __forceinline__ Divider make_divider(float s, bool plain) {
+  Divider d;
+  d.s = s;
+  d.plain = plain || !(s > 0x1p-100f && s < 0x1p100f);
+  d.yh = __uint_as_float(__float_as_uint(__builtin_amdgcn_rcpf(s)) - 2u);
+  const float e = __builtin_fmaf(-s, d.yh, 1.0f);
+  d.yl = __builtin_fmaf(e, e, e) * d.yh;
+  return d;
 }
 
-// 8 values / one scale -> 8 codes in two dwords, quotients rounded as by IEEE division.
-__device__ __forceinline__ v2i quant8(const float* v, float s, bool force_plain) {
-  const Divider d = make_divider(s, force_plain);
+// 8 values / one scale -> 8 codes in two dwords
+__device__ __forceinline__ v2i quant8(const float* v, const Divider& d) {
   float t[8];
-  auto pack = [&]() {
-    v2i o;
-    int w = pack2_fp8<false>(t[0], t[1], 0);
-    o[0] = pack2_fp8<true>(t[2], t[3], w);
-    w = pack2_fp8<false>(t[4], t[5], 0);
-    o[1] = pack2_fp8<true>(t[6], t[7], w);
-    return o;
-  };
   if (__builtin_expect(d.plain, 0)) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) t[i] = v[i] / s;
-    return pack();
-  }
+    for (int i = 0; i < 8; i++) t[i] = v[i] / d.s;
+  } else {
 #pragma unroll
-  for (int i = 0; i < 8; i++) t[i] = neg_div_by(v[i], d);
-  v2i o = pack();
-  o[0] ^= (int)0x80808080u;  // the quotients were negated: flip the sign bit of every code
-  o[1] ^= (int)0x80808080u;
+    for (int i = 0; i < 8; i++) t[i] = __builtin_fmaf(v[i], d.yh, v[i] * d.yl);
+  }
+  v2i o;
+  int w = pack2_fp8<false>(t[0], t[1], 0);
+  o[0] = pack2_fp8<true>(t[2], t[3], w);
+  w = pack2_fp8<false>(t[4], t[5], 0);
+  o[1] = pack2_fp8<true>(t[6], t[7], w);
   return o;
 }
 

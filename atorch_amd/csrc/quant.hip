@@ -4,7 +4,7 @@
 //
 // All of them stream HBM with 128-bit accesses; amax reductions over a 128-element tile run
 // inside one 16-lane DPP row.  Scales and codes are part of a bit-exact contract, so every
-// quotient is the correctly rounded one (the IEEE division or its checked three-instruction form).
+// quotient gives the code of the correctly rounded one (the IEEE division or its checked two-instruction form).
 #include "common.hpp"
 
 namespace aamd {
@@ -55,17 +55,16 @@ struct Raw8<F16> {
 
 // sigmoid on the hardware transcendental units, one v_exp_f32 and one v_rcp_f32 per value.  Both
 // flush results below the normal range, and 1 / (1 + e^-x) gets there for x below about -87 while
-// x times it is still a normal number, so everything is carried scaled by 2^16 (x r' stays finite for
-// |x| < 2^112):
-//   e' = 2^-16 e^-x (inf where e^-x itself overflows), r' = 1 / (2^-16 + e') = 2^16 sigmoid(x).
+// x times it is still a normal number, so the reciprocal is taken of the sum scaled by 2^-16
+// (x r' stays finite for |x| < 2^112):
+//   e = e^-x (inf where it overflows, 0 where it leaves the normal range), r' = 1 / (2^-16 + 2^-16 e)
+//   = 2^16 sigmoid(x).
 // silu(x) = (x r') 2^-16, sigmoid(x) = r' 2^-16.  A few fp32 ulps of error (more for |x| in the tens,
 // where x log2(e) itself is rounded), far below the bf16 rounding that follows; e^-x = inf gives
 // r' = 0 and silu = -0 as in fp32 arithmetic.
 __device__ __forceinline__ float sigmoid_scaled(float x) {
-  const float t = x * -1.4426950408889634f;
-  float e = __builtin_amdgcn_exp2f(t - 16.0f);
-  e = t >= 128.0f ? __builtin_inff() : e;  // where e^-x overflows in fp32 it does so here too
-  return __builtin_amdgcn_rcpf(0x1p-16f + e);
+  const float e = __builtin_amdgcn_exp2f(x * -1.4426950408889634f);
+  return __builtin_amdgcn_rcpf(__builtin_fmaf(e, 0x1p-16f, 0x1p-16f));
 }
 __device__ __forceinline__ float silu_from(float x, float r_scaled) { return (x * r_scaled) * 0x1p-16f; }
 
@@ -199,7 +198,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
                                                           int64_t M_out, uint8_t* __restrict__ q,
                                                           float* __restrict__ s, float eps, int64_t gate_off,
                                                           u16* __restrict__ h_out) {
-  // the three-instruction division is checked for bf16 values over scales of bf16 maxima only
+  // the short division is checked for bf16 values over scales of bf16 maxima only
   const bool plain_div = !kBf16Values<IN> || eps != 0.f;
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
   const int64_t base = (int64_t)blockIdx.x * (16 * U);
@@ -222,8 +221,9 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
   for (int u = 0; u < U; u++) {
     float v[8];
     raw[u].get(v);
-    const float sc = scale_from_amax(row16_max(amax8(v)), eps);
-    const v2i codes = quant8(v, sc, plain_div);
+    const Divider dv = make_scale(row16_max(amax8(v)), eps, plain_div);
+    const float sc = dv.s;
+    const v2i codes = quant8(v, dv);
     if (!valid[u]) continue;
     if (h_out != nullptr)  // the gated activation itself, for callers that keep it
       __builtin_nontemporal_store(pack8_bf16(v), reinterpret_cast<v4i*>(h_out + row[u] * cols + (int64_t)tc[u] * kTile + l * 8));
@@ -308,7 +308,7 @@ __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const f
     float col[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) col[i] = v[i][j];
-    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cs[j], plain_div);
+    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, make_divider(cs[j], plain_div));
   }
   store_staged_tile(tile_t, out, ld_out);
 }
@@ -319,7 +319,7 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
     u16* __restrict__ h_out, const u16* __restrict__ dh = nullptr, int64_t ld_dh = 0) {
-  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see quant8
+  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
   // SwiGLU backward: two teams of 256 threads per workgroup, one for the da tile and one for the db
   // tile of the same features, each with its own staging; both read a and dh at the same time, so
@@ -334,9 +334,23 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
   float* const cscale = cscales[team];
   __shared__ int slot;
 
-  int kc = blockIdx.x;
-  const int pt = blockIdx.y;
-  if constexpr (TEAMS == 2) kc = team * (nt / 2) + blockIdx.x;  // da tiles first, then db tiles
+  // Workgroups go to the eight XCDs in turn, and the row-wise scales of a tile are 128 single floats, one
+  // per row: with tile = workgroup index, the eight floats of a 32-byte sector would come from eight
+  // different L2 caches and reach memory as eight partial writes.  The index is therefore re-dealt so
+  // that eight consecutive workgroups of one XCD take eight consecutive column tiles of one token tile.
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  {
+    const uint32_t ntx = gridDim.x, per_row = ntx >> 3;
+    const uint32_t lin = by * ntx + bx, chunks = gridDim.y * per_row;
+    if ((ntx & 7) == 0 && lin < (chunks & ~7u) * 8) {
+      const uint32_t j = lin >> 3, chunk = (j & ~7u) + (lin & 7);
+      by = chunk / per_row;
+      bx = (chunk - by * per_row) * 8 + (j & 7);
+    }
+  }
+  const int pt = (int)by;
+  int kc = (int)bx;
+  if constexpr (TEAMS == 2) kc = team * (nt / 2) + (int)bx;  // da tiles first, then db tiles
   const int g = find_group(tile_off, E, pt, &slot);
   if (g >= E) return;
   const int64_t cols = (int64_t)nt * kTile;
@@ -366,9 +380,10 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
     if (h_out != nullptr && gr * 8 + i < mvalid)
       __builtin_nontemporal_store(pack8_bf16(v[i]), reinterpret_cast<v4i*>(h_out + (m0 + gr * 8 + i) * cols + (int64_t)kc * kTile + c * 8));
     if (q != nullptr) {
-      const float sc = scale_from_amax(row16_max(amax8(v[i])), eps);
+      const Divider dv = make_scale(row16_max(amax8(v[i])), eps, plain_div);
+      const float sc = dv.s;
       const int r = gr * 8 + i;
-      const v2i codes = quant8(v[i], sc, plain_div);
+      const v2i codes = quant8(v[i], dv);
       if (r < mvalid) {
         __builtin_nontemporal_store(codes, reinterpret_cast<v2i*>(q + (m0 + r) * cols + (int64_t)kc * kTile + c * 8));
         if (c == 0) s[(m0 + r) * nt + kc] = sc;
@@ -383,7 +398,7 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
     float m = part[0][team_tid()];
 #pragma unroll
     for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][team_tid()]);
-    const float sc = scale_from_amax(m, eps);
+    const float sc = make_scale(m, eps, plain_div).s;
     cscale[team_tid()] = sc;
     s_t[(int64_t)pt * cols + (int64_t)kc * kTile + team_tid()] = sc;
   }
@@ -420,7 +435,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
                                                             uint8_t* __restrict__ q, float* __restrict__ s,
                                                             uint8_t* __restrict__ q_t, float* __restrict__ s_t,
                                                             float eps) {
-  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see quant8
+  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   __shared__ float part[16];
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
   const int kb = blockIdx.x, nb = blockIdx.y, e = blockIdx.z;
@@ -437,7 +452,8 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < 16; i++) m = fmaxf(m, part[i]);
-  const float sc = scale_from_amax(m, eps);
+  const Divider dv = make_scale(m, eps, plain_div);
+  const float sc = dv.s;
   if (threadIdx.x == 0) {
     s[((int64_t)e * nnb + nb) * nkb + kb] = sc;
     if (s_t != nullptr) s_t[((int64_t)e * nkb + kb) * nnb + nb] = sc;
@@ -446,7 +462,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
   v2i codes[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
-    codes[i] = quant8(v[i], sc, plain_div);
+    codes[i] = quant8(v[i], dv);
     __builtin_nontemporal_store(codes[i], reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8));
   }
   if (q_t != nullptr) {

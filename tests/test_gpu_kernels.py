@@ -496,6 +496,41 @@ def test_fp8_gemm_tile_scaled_b_large_tiles(dev, out_dtype):
     assert torch.equal(c, c_small)
 
 
+@pytest.mark.parametrize("K", [512, 1024, 1536, 2560, 1152], ids=lambda k: f"K{k}")
+def test_grouped_gemm_nt_scale_batches_of_the_large_tiles(dev, K):
+    """The 256x256 configuration takes its scales in batches of eight contraction blocks: exactly one
+    batch (K = 1024), a last batch shifted back to end at the last block (1536, 2560), and contractions
+    that cannot be batched (512: fewer than eight blocks; 1152: not a multiple of four blocks), which the
+    launcher gives to the 128x128 configuration.  Ragged groups with an empty one, a partial last R tile
+    (N = 640), bias; against the float64 definition on the device and, bit for bit, against the pinned
+    128x128 configuration, which adds the same products in the same order."""
+    from atorch_amd import kernels
+
+    E, N = 4, 640
+    splits = [700, 0, 1301, 255]
+    M = sum(splits)
+    x = randn_bf16((M, K), 51).to(dev)
+    w = randn_bf16((E, N, K), 52, std=0.02).to(dev)
+    bias = randn_bf16((E, N), 53).to(dev)
+    qx, sx = kernels.tile_quant(x)
+    qw, sw, _, _ = kernels.block_quant_batched(w)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    with kernels.gemm_options(tile=1):
+        y = kernels.grouped_gemm_nt(qx, sx, qw, sw, goff, out_dtype=torch.float32, bias=bias)
+    with kernels.gemm_options(tile=0):
+        y_small = kernels.grouped_gemm_nt(qx, sx, qw, sw, goff, out_dtype=torch.float32, bias=bias)
+    assert torch.equal(y, y_small)
+    xd = _deq_tile(qx, sx).double()
+    ref = torch.zeros(M, N, dtype=torch.float64, device=dev)
+    off = 0
+    for e, m in enumerate(splits):
+        if m:
+            wd = qw[e].float() * sw[e].repeat_interleave(TILE, -2).repeat_interleave(TILE, -1)
+            ref[off : off + m] = xd[off : off + m] @ wd.double().t() + bias[e].double()
+        off += m
+    assert rel_err(y.cpu(), ref.float().cpu()) <= GEMM_TOL_F32
+
+
 @pytest.mark.parametrize("tile", [0, 1], ids=["small", "large"])
 def test_grouped_gemm_wgrad_pinned_tile_configurations(dev, tile):
     """Both tile configurations of the weight-gradient GEMM (the library picks one by shape) on ragged
