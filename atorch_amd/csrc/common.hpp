@@ -134,8 +134,8 @@ __device__ __forceinline__ int pack2_fp8(float a, float b, int old) {
 //     That is no proof of a correctly rounded quotient: the scheme is used where every case has been
 //     enumerated and gives the code of the plain division: all pairs of a bf16 value and a bf16 maximum,
 //     about 10^9.
-// Maxima outside 2^-90 .. 2^100 (zero aside) take the plain path, where a residual or a reciprocal could
-// leave the normal range.
+// Maxima outside 2^-90 .. 2^100 (zero among them) take the plain path, where a residual or a reciprocal
+// could leave the normal range.
 struct Divider {
   float s, yh, yl;
   bool plain;
@@ -143,7 +143,9 @@ struct Divider {
 __device__ __forceinline__ Divider make_scale(float amax, float eps, bool plain) {
   const float a = fmaxf(amax, eps);
   Divider d;
-  d.plain = plain || !(a < 0x1p100f) || (a < 0x1p-90f && a > 0.f);
+  // 2^-90 <= a < 2^100 as one unsigned comparison of the bit patterns (a is not negative; zero, NaN and
+  // infinity fall outside)
+  d.plain = plain || __float_as_uint(a) - 0x12800000u >= 0x71800000u - 0x12800000u;
   if (__builtin_expect(d.plain, 0)) {
     const float s = a / kFp8Max;
     d.s = s == 0.f ? 1.f : s;
@@ -152,41 +154,34 @@ __device__ __forceinline__ Divider make_scale(float amax, float eps, bool plain)
     constexpr float y = 1.0f / kFp8Max;
     const float q = a * y;
     const float r = __builtin_fmaf(-kFp8Max, q, a);
-    const float s = __builtin_fmaf(r, y, q);
-    d.s = s == 0.f ? 1.f : s;
+    d.s = __builtin_fmaf(r, y, q);  // not zero: a >= 2^-90
     d.yh = __uint_as_float(__float_as_uint(__builtin_amdgcn_rcpf(d.s)) - 2u);
     const float e = __builtin_fmaf(-d.s, d.yh, 1.0f);
     d.yl = __builtin_fmaf(e, e, e) * d.yh;
   }
   return d;
 }
-// the divider of a scale that make_scale produced elsewhere (`plain` as it was given there)
-__device__ __forceinline__ Divider make_divider(float s, bool plain) {
-  Divider d;
-  d.s = s;
-  d.plain = plain || !(s > 0x1p-100f && s < 0x1p100f);
-  d.yh = __uint_as_float(__float_as_uint(__builtin_amdgcn_rcpf(s)) - 2u);
-  const float e = __builtin_fmaf(-s, d.yh, 1.0f);
-  d.yl = __builtin_fmaf(e, e, e) * d.yh;
-  return d;
-}
-
-// 8 values / one scale -> 8 codes in two dwords
-__device__ __forceinline__ v2i quant8(const float* v, const Divider& d) {
-  float t[8];
-  if (__builtin_expect(d.plain, 0)) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) t[i] = v[i] / d.s;
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; i++) t[i] = __builtin_fmaf(v[i], d.yh, v[i] * d.yl);
-  }
+__device__ __forceinline__ v2i pack8_fp8(const float* t) {
   v2i o;
   int w = pack2_fp8<false>(t[0], t[1], 0);
   o[0] = pack2_fp8<true>(t[2], t[3], w);
   w = pack2_fp8<false>(t[4], t[5], 0);
   o[1] = pack2_fp8<true>(t[6], t[7], w);
   return o;
+}
+// the plain path, out of line: a hundred instructions that the kernels of bf16 inputs almost never run
+__device__ __attribute__((noinline)) v2i quant8_plain(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                                                      float v7, float s) {
+  const float t[8] = {v0 / s, v1 / s, v2 / s, v3 / s, v4 / s, v5 / s, v6 / s, v7 / s};
+  return pack8_fp8(t);
+}
+// 8 values / one scale -> 8 codes in two dwords
+__device__ __forceinline__ v2i quant8(const float* v, const Divider& d) {
+  if (__builtin_expect(d.plain, 0)) return quant8_plain(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], d.s);
+  float t[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) t[i] = __builtin_fmaf(v[i], d.yh, v[i] * d.yl);
+  return pack8_fp8(t);
 }
 
 __device__ __forceinline__ float amax8(const float* v) {

@@ -16,7 +16,7 @@ constexpr int kMaxTopk = 64;
 // YT: element type of the permuted rows (BF16 or F32); the result has the promoted type of rows and
 // probs (fp32 rows, or fp32 probs, give fp32).
 template <typename YT, int PD>
-__global__ __launch_bounds__(256) void unpermute_combine_kernel(const typename YT::elem* __restrict__ y, int64_t M, int H8,
+__global__ __launch_bounds__(512) void unpermute_combine_kernel(const typename YT::elem* __restrict__ y, int64_t M, int H8,
                                                                 const int32_t* __restrict__ row_map,
                                                                 const void* __restrict__ probs, int topk,
                                                                 void* __restrict__ out) {
@@ -545,7 +545,16 @@ extern "C" int aamd_unpermute_combine(const void* y, int y_dtype, int64_t M, int
   AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs != nullptr, "unpermute_combine: probs missing");
   AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0, "unpermute_combine: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)T), block(256);
+  // one workgroup per token, one 16-byte chunk of the row per lane and trip: the workgroup size that
+  // leaves the fewest lanes idle in the last trip (7168 columns of bf16: 448 lanes, two full trips)
+  const int64_t chunks = H / (y_dtype == AAMD_BF16 ? 8 : 4);
+  int threads = 256;
+  int64_t waste = (chunks + 255) / 256 * 256 - chunks;
+  for (int b = 512; b >= 128; b -= 64) {
+    const int64_t w = (chunks + b - 1) / b * b - chunks;
+    if (w < waste) { waste = w; threads = b; }
+  }
+  dim3 grid((unsigned)T), block((unsigned)threads);
   if (y_dtype == AAMD_BF16) {
     const int H8 = (int)(H / 8);
     if (probs_dtype == AAMD_BF16)

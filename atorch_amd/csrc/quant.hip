@@ -12,21 +12,36 @@ namespace aamd {
 // ---------------------------------------------------------------------------------------
 // tile loaders: 8 consecutive elements per lane
 // ---------------------------------------------------------------------------------------
+// 16 bytes at a byte offset from a base pointer.  With a base that is the same in every lane the
+// address is a scalar register pair plus a 32-bit lane offset: no 64-bit arithmetic per access.
+template <typename T>
+__device__ __forceinline__ v4i ld16(const T* base, uint32_t boff) {
+  return *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(base) + boff);
+}
+template <typename T>
+__device__ __forceinline__ v4i ld16_nt(const T* base, uint32_t boff) {
+  return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(base) + boff));
+}
+template <typename V, typename T>
+__device__ __forceinline__ void st_nt(T* base, uint32_t boff, V val) {
+  __builtin_nontemporal_store(val, reinterpret_cast<V*>(reinterpret_cast<char*>(base) + boff));
+}
+
 template <typename IN>
 struct Raw8;
 template <>
 struct Raw8<BF16> {
   v4i a;
-  __device__ __forceinline__ void load(const u16* p, int64_t) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
+  __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t) { a = ld16_nt(p, boff); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const { unpack8(a, v); }
 };
 template <>
 struct Raw8<F32> {
   v4i a, b;
-  __device__ __forceinline__ void load(const float* p, int64_t) {
-    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
-    b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p) + 1);
+  __device__ __forceinline__ void load(const float* p, uint32_t boff, int64_t) {
+    a = ld16_nt(p, boff);
+    b = ld16_nt(p + 4, boff);
   }
   __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const {
@@ -41,7 +56,7 @@ struct Raw8<F32> {
 template <>
 struct Raw8<F16> {
   v4i a;
-  __device__ __forceinline__ void load(const u16* p, int64_t) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
+  __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t) { a = ld16_nt(p, boff); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const {
 #pragma unroll
@@ -73,9 +88,9 @@ __device__ __forceinline__ float silu_from(float x, float r_scaled) { return (x 
 template <>
 struct Raw8<GLU> {
   v4i a, b;
-  __device__ __forceinline__ void load(const u16* p, int64_t gate_off) {
-    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
-    b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p + gate_off));
+  __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t gate_off) {
+    a = ld16_nt(p, boff);
+    b = ld16_nt(p + gate_off, boff);
   }
   __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const {
@@ -98,14 +113,16 @@ struct Raw8<GLU> {
 // eight elements of da or of db.
 struct GluBwd8 {
   v4i a, b, d;
-  __device__ __forceinline__ void load(const u16* pa, int64_t gate_off, const u16* pd, bool want_db) {
-    a = *reinterpret_cast<const v4i*>(pa);  // a and dh are read by both teams: plain loads, kept in the caches
-    d = *reinterpret_cast<const v4i*>(pd);
-    if (!want_db) b = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(pa + gate_off));
+  template <bool WANT_DB>
+  __device__ __forceinline__ void load(const u16* pa, uint32_t boff, int64_t gate_off, const u16* pd, uint32_t boff_d) {
+    a = ld16(pa, boff);  // a and dh are read by both teams: plain loads, kept in the caches
+    d = ld16(pd, boff_d);
+    if constexpr (!WANT_DB) b = ld16_nt(pa + gate_off, boff);
     else b = v4i{0, 0, 0, 0};
   }
   __device__ __forceinline__ void zero() { a = b = d = v4i{0, 0, 0, 0}; }
-  __device__ __forceinline__ void get(float* v, bool want_db) const {
+  template <bool WANT_DB>
+  __device__ __forceinline__ void get(float* v) const {
     float fa[8], fb[8], fd[8];
     unpack8(a, fa);
     unpack8(b, fb);
@@ -114,7 +131,7 @@ struct GluBwd8 {
     for (int i = 0; i < 8; i += 2) {
       float r0, r1;
       const float rs0 = sigmoid_scaled(fa[i]), rs1 = sigmoid_scaled(fa[i + 1]);
-      if (want_db) {
+      if constexpr (WANT_DB) {
         const uint32_t sl = pack_bf16x2(silu_from(fa[i], rs0), silu_from(fa[i + 1], rs1));
         r0 = fd[i] * __uint_as_float(sl << 16);
         r1 = fd[i + 1] * __uint_as_float(sl & 0xffff0000u);
@@ -136,7 +153,7 @@ struct GluBwd8 {
 template <>
 struct Raw8<GELU> {
   v4i a;
-  __device__ __forceinline__ void load(const u16* p, int64_t) { a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p)); }
+  __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t) { a = ld16_nt(p, boff); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const {
     float x[8];
@@ -154,9 +171,9 @@ struct Raw8<GELU> {
 template <>
 struct Raw8<GELUB> {
   v4i a, d;
-  __device__ __forceinline__ void load(const u16* p, int64_t dh_off) {
-    a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
-    d = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p + dh_off));
+  __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t dh_off) {
+    a = ld16_nt(p, boff);
+    d = ld16_nt(p + dh_off, boff);
   }
   __device__ __forceinline__ void zero() { a = d = v4i{0, 0, 0, 0}; }
   __device__ __forceinline__ void get(float* v) const {
@@ -215,7 +232,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     if (!valid[u]) tile = total_tiles - 1;
     row[u] = tile / nt;
     tc[u] = (int)(tile - row[u] * nt);
-    raw[u].load(x + row[u] * ldx + (int64_t)tc[u] * kTile + l * 8, gate_off);
+    raw[u].load(x + row[u] * ldx + (int64_t)tc[u] * kTile + l * 8, 0u, gate_off);
   }
 #pragma unroll
   for (int u = 0; u < U; u++) {
@@ -248,19 +265,23 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
 // 256 threads, thread (gr = tid/16, c = tid%16) holds rows gr*8 .. gr*8+7, columns c*8 .. c*8+7.
 // ---------------------------------------------------------------------------------------
 constexpr int kTLd = kTile + 16;  // LDS row stride (bytes) of the transposed code tile
+// 128 rows of a tile are addressed with 32-bit byte offsets: row strides (elements, at most 4 bytes each) stay below this
+constexpr int64_t kMaxTileLd = (int64_t)1 << 22;
 // thread index inside a 256-thread tile team (a workgroup is one team, or two for the SwiGLU backward)
 __device__ __forceinline__ int team_tid() { return threadIdx.x & 255; }
 
-template <typename IN>
-__device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, int64_t ldx, int rows_valid,
+// `x` is the tile's origin, the same in every lane; FULL: all 128 rows are valid
+template <typename IN, bool FULL>
+__device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int rows_valid,
                                           float (&v)[8][8], int64_t gate_off = 0) {
   const int gr = team_tid() >> 4, c = team_tid() & 15;
+  constexpr uint32_t kEl = sizeof(typename IN::elem);
+  const uint32_t off0 = ((uint32_t)(gr * 8) * ldx + (uint32_t)c * 8) * kEl;
   Raw8<IN> raw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
-    const int r = gr * 8 + i;
-    if (r < rows_valid)
-      raw[i].load(x + (int64_t)r * ldx + c * 8, gate_off);
+    if (FULL || gr * 8 + i < rows_valid)
+      raw[i].load(x, off0 + (uint32_t)i * ldx * kEl, gate_off);
     else
       raw[i].zero();
   }
@@ -268,49 +289,115 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
   for (int i = 0; i < 8; i++) raw[i].get(v[i]);
 }
 
-// the same register tile of da (want_db false) or db for feature columns [f0, f0 + 128)
-__device__ __forceinline__ void load_tile_glu_bwd(const u16* __restrict__ fc1, int64_t ld, int64_t gate_off,
-                                                  const u16* __restrict__ dh, int64_t ld_dh, bool want_db,
-                                                  int rows_valid, float (&v)[8][8]) {
+// the same register tile of da (WANT_DB false) or db of one feature tile (fc1 and dh at the tile's origin)
+template <bool WANT_DB, bool FULL>
+__device__ __forceinline__ void load_tile_glu_bwd(const u16* __restrict__ fc1, uint32_t ld, int64_t gate_off,
+                                                  const u16* __restrict__ dh, uint32_t ld_dh, int rows_valid,
+                                                  float (&v)[8][8]) {
   const int gr = team_tid() >> 4, c = team_tid() & 15;
+  const uint32_t off0 = ((uint32_t)(gr * 8) * ld + (uint32_t)c * 8) * 2, off0d = ((uint32_t)(gr * 8) * ld_dh + (uint32_t)c * 8) * 2;
   GluBwd8 raw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
-    const int r = gr * 8 + i;
-    if (r < rows_valid)
-      raw[i].load(fc1 + (int64_t)r * ld + c * 8, gate_off, dh + (int64_t)r * ld_dh + c * 8, want_db);
+    if (FULL || gr * 8 + i < rows_valid)
+      raw[i].template load<WANT_DB>(fc1, off0 + (uint32_t)i * ld * 2, gate_off, dh, off0d + (uint32_t)i * ld_dh * 2);
     else
       raw[i].zero();
   }
 #pragma unroll
-  for (int i = 0; i < 8; i++) raw[i].get(v[i], want_db);
+  for (int i = 0; i < 8; i++) raw[i].template get<WANT_DB>(v[i]);
 }
 
 // the staged 128 x 128 code tile written as rows of 128 bytes, one 16-byte store per lane
-__device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t* __restrict__ out, int64_t ld_out) {
+// (`out`: the tile's origin, the same in every lane; 128 ld_out < 2^32)
+__device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t* __restrict__ out, uint32_t ld_out) {
   __syncthreads();
 #pragma unroll
   for (int n = 0; n < 4; n++) {
     const int idx = team_tid() + 256 * n;
     const int r = idx >> 3, ch = idx & 7;
-    __builtin_nontemporal_store(*reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16),
-                                reinterpret_cast<v4i*>(out + (int64_t)r * ld_out + ch * 16));
+    st_nt(out, (uint32_t)r * ld_out + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16));
   }
 }
 
 // codes of the 8x8 register block, transposed through LDS, written as rows of 128 bytes:
 // out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
-__device__ __forceinline__ void store_transposed(const float (&v)[8][8], const float* cs, uint8_t* tile_t,
-                                                 uint8_t* __restrict__ out, int64_t ld_out, bool plain_div) {
+__device__ __forceinline__ void store_transposed(const float (&v)[8][8], const Divider* cdiv, uint8_t* tile_t,
+                                                 uint8_t* __restrict__ out, uint32_t ld_out) {
   const int gr = team_tid() >> 4, c = team_tid() & 15;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
     float col[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) col[i] = v[i][j];
-    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, make_divider(cs[j], plain_div));
+    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cdiv[j * 16]);
   }
   store_staged_tile(tile_t, out, ld_out);
+}
+
+// One 128 x 128 tile of the dual quantiser: token tile pt of group g, column tile kc.  Everything that
+// locates the tile is the same in every lane, so each access is a scalar base plus a 32-bit lane offset
+// (the launchers bound the row strides so that 128 rows stay below 2^32 bytes).
+template <typename IN, bool WANT_DB, bool FULL>
+__device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int nt, int64_t m0,
+                                          int mvalid, int pt, int kc, uint8_t* __restrict__ q, float* __restrict__ s,
+                                          uint8_t* __restrict__ q_t, float* __restrict__ s_t, uint32_t ld_t, float eps,
+                                          int64_t gate_off, u16* __restrict__ h_out, const u16* __restrict__ dh,
+                                          uint32_t ld_dh, uint8_t* tile_t, Divider* cdiv) {
+  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
+  float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
+  const int64_t cols = (int64_t)nt * kTile;
+  const int gr = team_tid() >> 4, c = team_tid() & 15;
+
+  float v[8][8];
+  if constexpr (std::is_same<IN, GLUB>::value) {
+    const int half = nt / 2;  // output column tiles [0, half) are da, [half, nt) are db
+    const int64_t f0 = (int64_t)(WANT_DB ? kc - half : kc) * kTile;
+    load_tile_glu_bwd<WANT_DB, FULL>(x + m0 * ldx + f0, ldx, gate_off, dh + m0 * ld_dh + f0, ld_dh, mvalid, v);
+  } else {
+    load_tile<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
+  }
+
+  // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
+  u16* const hb = h_out ? h_out + m0 * cols + (int64_t)kc * kTile : nullptr;
+  uint8_t* const qb = q ? q + m0 * cols + (int64_t)kc * kTile : nullptr;
+  float* const sb = q ? s + m0 * nt + kc : nullptr;
+  const uint32_t ucols = (uint32_t)cols;
+  float cm[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) cm[j] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const uint32_t r = (uint32_t)(gr * 8 + i);
+    const bool live = FULL || (int)r < mvalid;
+    if (hb != nullptr && live) st_nt(hb, (r * ucols + (uint32_t)c * 8) * 2, pack8_bf16(v[i]));
+    if (qb != nullptr) {
+      const Divider dv = make_scale(row16_max(amax8(v[i])), eps, plain_div);
+      const v2i codes = quant8(v[i], dv);
+      if (live) {
+        st_nt(qb, r * ucols + (uint32_t)c * 8, codes);
+        if (c == 0) *reinterpret_cast<float*>(reinterpret_cast<char*>(sb) + r * (uint32_t)nt * 4) = dv.s;
+      }
+    }
+  }
+  // column amax over the 128 tokens of the tile (two rows per three-operand maximum)
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) cm[j] = fmaxf(fmaxf(cm[j], fabsf(v[i][j])), fabsf(v[i + 1][j]));
+    part[gr][c * 8 + j] = cm[j];
+  }
+  __syncthreads();
+  if (team_tid() < kTile) {
+    float m = part[0][team_tid()];
+#pragma unroll
+    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][team_tid()]);
+    const Divider dv = make_scale(m, eps, plain_div);
+    cdiv[(team_tid() & 7) * 16 + (team_tid() >> 3)] = dv;  // [column % 8][column / 8]: lanes of a row read 16 neighbours
+    (s_t + (int64_t)pt * cols + (int64_t)kc * kTile)[team_tid()] = dv.s;
+  }
+  __syncthreads();
+  store_transposed(v, cdiv + c, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
 }
 
 template <typename IN>
@@ -319,19 +406,15 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
     u16* __restrict__ h_out, const u16* __restrict__ dh = nullptr, int64_t ld_dh = 0) {
-  const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
   // SwiGLU backward: two teams of 256 threads per workgroup, one for the da tile and one for the db
   // tile of the same features, each with its own staging; both read a and dh at the same time, so
   // the second read is served by the caches and HBM sees every input once
   constexpr int TEAMS = std::is_same<IN, GLUB>::value ? 2 : 1;
-  const int team = TEAMS == 2 ? (int)(threadIdx.x >> 8) : 0;
+  const int team = TEAMS == 2 ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) : 0;
   __shared__ __attribute__((aligned(16))) uint8_t tile_ts[TEAMS][kTile * kTLd];
   static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_ts[0]), "the column maxima fit in the staging region");
-  uint8_t* const tile_t = tile_ts[team];
-  float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
-  __shared__ float cscales[TEAMS][kTile];
-  float* const cscale = cscales[team];
+  __shared__ Divider cdivs[TEAMS][kTile];  // scale and divider of every column of the tile
   __shared__ int slot;
 
   // Workgroups go to the eight XCDs in turn, and the row-wise scales of a tile are 128 single floats, one
@@ -351,62 +434,29 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
   const int pt = (int)by;
   int kc = (int)bx;
   if constexpr (TEAMS == 2) kc = team * (nt / 2) + (int)bx;  // da tiles first, then db tiles
-  const int g = find_group(tile_off, E, pt, &slot);
+  const int g = __builtin_amdgcn_readfirstlane(find_group(tile_off, E, pt, &slot));
   if (g >= E) return;
-  const int64_t cols = (int64_t)nt * kTile;
   const int64_t m0 = goff[g] + (int64_t)(pt - tile_off[g]) * kTile;
   const int64_t left = goff[g + 1] - m0;
   const int mvalid = left < kTile ? (int)left : kTile;
-  const int gr = team_tid() >> 4, c = team_tid() & 15;
+  uint8_t* const tile_t = tile_ts[team];
+  Divider* const cdiv = cdivs[team];
 
-  float v[8][8];
-  if constexpr (std::is_same<IN, GLUB>::value) {
-    const int half = nt / 2;  // output column tiles [0, half) are da, [half, nt) are db
-    const bool want_db = kc >= half;
-    const int64_t f0 = (int64_t)(want_db ? kc - half : kc) * kTile;
-    load_tile_glu_bwd(x + m0 * ldx + f0, ldx, gate_off, dh + m0 * ld_dh + f0, ld_dh, want_db, mvalid, v);
+  auto run = [&](auto WANT_DB, auto FULL) {
+    dual_tile<IN, decltype(WANT_DB)::value, decltype(FULL)::value>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t,
+                                                                   (uint32_t)ld_t, eps, gate_off, h_out, dh,
+                                                                   (uint32_t)ld_dh, tile_t, cdiv);
+  };
+  auto run_full = [&](auto WANT_DB) {
+    if (mvalid == kTile) run(WANT_DB, std::true_type{});
+    else run(WANT_DB, std::false_type{});
+  };
+  if constexpr (TEAMS == 2) {
+    if (team == 0) run_full(std::false_type{});
+    else run_full(std::true_type{});
   } else {
-    load_tile<IN>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
+    run_full(std::false_type{});
   }
-
-  // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
-  float cm[8];
-#pragma unroll
-  for (int j = 0; j < 8; j++) cm[j] = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) cm[j] = fmaxf(cm[j], fabsf(v[i][j]));
-    if (h_out != nullptr && gr * 8 + i < mvalid)
-      __builtin_nontemporal_store(pack8_bf16(v[i]), reinterpret_cast<v4i*>(h_out + (m0 + gr * 8 + i) * cols + (int64_t)kc * kTile + c * 8));
-    if (q != nullptr) {
-      const Divider dv = make_scale(row16_max(amax8(v[i])), eps, plain_div);
-      const float sc = dv.s;
-      const int r = gr * 8 + i;
-      const v2i codes = quant8(v[i], dv);
-      if (r < mvalid) {
-        __builtin_nontemporal_store(codes, reinterpret_cast<v2i*>(q + (m0 + r) * cols + (int64_t)kc * kTile + c * 8));
-        if (c == 0) s[(m0 + r) * nt + kc] = sc;
-      }
-    }
-  }
-  // column amax over the 128 tokens of the tile
-#pragma unroll
-  for (int j = 0; j < 8; j++) part[gr][c * 8 + j] = cm[j];
-  __syncthreads();
-  if (team_tid() < kTile) {
-    float m = part[0][team_tid()];
-#pragma unroll
-    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][team_tid()]);
-    const float sc = make_scale(m, eps, plain_div).s;
-    cscale[team_tid()] = sc;
-    s_t[(int64_t)pt * cols + (int64_t)kc * kTile + team_tid()] = sc;
-  }
-  __syncthreads();
-  float cs[8];
-#pragma unroll
-  for (int j = 0; j < 8; j++) cs[j] = cscale[c * 8 + j];
-  store_transposed(v, cs, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t, plain_div);
 }
 
 // The 8x8 byte matrix held as eight rows of two dwords, transposed with byte permutes: cols[j]
@@ -443,7 +493,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
   const int gr = threadIdx.x >> 4, c = threadIdx.x & 15;
 
   float v[8][8];
-  load_tile<IN>(w + e * expert_stride + (int64_t)nb * kTile * K + (int64_t)kb * kTile, K, kTile, v);
+  load_tile<IN, true>(w + e * expert_stride + (int64_t)nb * kTile * K + (int64_t)kb * kTile, (uint32_t)K, kTile, v);
   float m = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; i++) m = fmaxf(m, amax8(v[i]));
@@ -463,7 +513,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     codes[i] = quant8(v[i], dv);
-    __builtin_nontemporal_store(codes[i], reinterpret_cast<v2i*>(qe + (int64_t)(gr * 8 + i) * K + c * 8));
+    st_nt(qe, (uint32_t)(gr * 8 + i) * (uint32_t)K + (uint32_t)c * 8, codes[i]);
   }
   if (q_t != nullptr) {
     // one scale for the whole block: the transposed copy holds the same codes, so the 8x8 block of
@@ -472,7 +522,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
     transpose8x8_bytes(codes, cols);
 #pragma unroll
     for (int j = 0; j < 8; j++) *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = cols[j];
-    store_staged_tile(tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, N);
+    store_staged_tile(tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, (uint32_t)N);
   }
 }
 
@@ -607,7 +657,8 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
   AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "quant_dual: unsupported dtype %d", x_dtype);
   AAMD_REQUIRE(M >= 0 && cols >= 0 && cols % kTile == 0, "quant_dual: cols=%lld must be a multiple of 128",
                (long long)cols);
-  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "quant_dual: bad ldx=%lld", (long long)ldx);
+  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0 && ldx < kMaxTileLd, "quant_dual: bad ldx=%lld", (long long)ldx);
+  AAMD_REQUIRE(ld_t < kMaxTileLd, "quant_dual: ld_t=%lld too large", (long long)ld_t);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "quant_dual: group_offsets / tile_ws required");
   AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
   AAMD_REQUIRE((q == nullptr) == (s == nullptr), "quant_dual: q and s go together");
@@ -663,7 +714,7 @@ extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, 
                                                     void* h_out, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
                                                     int64_t ld_t, void* stream) {
   AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "swiglu_quant_dual: F=%lld must be a multiple of 128", (long long)F);
-  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0, "swiglu_quant_dual: bad ld=%lld", (long long)ld);
+  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld < kMaxTileLd && ld_t < kMaxTileLd, "swiglu_quant_dual: bad ld=%lld", (long long)ld);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "swiglu_quant_dual: group_offsets / tile_ws required");
   AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "swiglu_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
   AAMD_REQUIRE((q == nullptr) == (s == nullptr), "swiglu_quant_dual: q and s go together");
@@ -711,7 +762,7 @@ extern "C" int aamd_gelu_quant_1x128_dual_grouped(const void* x, const void* dh,
                                                   uint8_t* q, float* s, uint8_t* q_t, float* s_t, int64_t ld_t,
                                                   void* stream) {
   AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "gelu_quant_dual: F=%lld must be a multiple of 128", (long long)F);
-  AAMD_REQUIRE(ld >= F && ld % 8 == 0, "gelu_quant_dual: bad ld=%lld", (long long)ld);
+  AAMD_REQUIRE(ld >= F && ld % 8 == 0 && ld < kMaxTileLd && ld_t < kMaxTileLd, "gelu_quant_dual: bad ld=%lld", (long long)ld);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "gelu_quant_dual: group_offsets / tile_ws required");
   AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "gelu_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
   AAMD_REQUIRE((q == nullptr) == (s == nullptr), "gelu_quant_dual: q and s go together");
@@ -745,7 +796,8 @@ extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t 
                                                         int32_t* tile_ws, void* g_out, uint8_t* q, float* s,
                                                         uint8_t* q_t, float* s_t, int64_t ld_t, void* stream) {
   AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "swiglu_bwd_quant_dual: F=%lld must be a multiple of 128", (long long)F);
-  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld_dh >= F && ld_dh % 8 == 0, "swiglu_bwd_quant_dual: bad ld=%lld / ld_dh=%lld",
+  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld_dh >= F && ld_dh % 8 == 0 && ld < kMaxTileLd && ld_dh < kMaxTileLd && ld_t < kMaxTileLd,
+               "swiglu_bwd_quant_dual: bad ld=%lld / ld_dh=%lld",
                (long long)ld, (long long)ld_dh);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "swiglu_bwd_quant_dual: group_offsets / tile_ws required");
   AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "swiglu_bwd_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
@@ -777,6 +829,7 @@ extern "C" int aamd_quant_128x128(const void* w, int w_dtype, int64_t E, int64_t
   AAMD_REQUIRE(E >= 0 && N >= 0 && K >= 0 && N % kTile == 0 && K % kTile == 0,
                "quant_128x128: N=%lld and K=%lld must be multiples of 128", (long long)N, (long long)K);
   AAMD_REQUIRE((q_t == nullptr) == (s_t == nullptr), "quant_128x128: q_t and s_t go together");
+  AAMD_REQUIRE(N < kMaxTileLd && K < kMaxTileLd, "quant_128x128: N=%lld or K=%lld too large", (long long)N, (long long)K);
   if (E == 0 || N == 0 || K == 0) return AAMD_OK;
   AAMD_REQUIRE(w && q && s, "quant_128x128: null pointer");
   AAMD_REQUIRE(expert_stride >= N * K && expert_stride % 8 == 0, "quant_128x128: bad expert stride");
