@@ -56,12 +56,6 @@ struct BF16 {
 struct GLU {
   typedef u16 elem;
 };
-// Backward of the same unit: rows [a | b] plus the gradient dh of h; the element read at column c
-// of the [da | db] row is da = bf16(bf16(dh*b) * sig(a) * (1 + a*(1 - sig(a)))) or
-// db = bf16(dh * bf16(silu(a))), what autograd makes of the two torch ops on bf16 tensors.
-struct GLUB {
-  typedef u16 elem;
-};
 // bf16 values x read as h = bf16(gelu(x)), gelu(x) = x/2 (1 + erf(x / sqrt 2)) in fp32: the default
 // activation of the expert MLP (grouped_gemm_moe.py:449, torch.nn.functional.gelu).
 struct GELU {
@@ -175,9 +169,19 @@ __device__ __attribute__((noinline)) v2i quant8_plain(float v0, float v1, float 
   const float t[8] = {v0 / s, v1 / s, v2 / s, v3 / s, v4 / s, v5 / s, v6 / s, v7 / s};
   return pack8_fp8(t);
 }
-// 8 values / one scale -> 8 codes in two dwords
+// 8 values / one scale -> 8 codes in two dwords.  CALL_PLAIN: the plain path is a function call (values that live
+// across a call sit in the callee-saved half of the register file, which costs a kernel with many live values
+// its occupancy: such kernels keep the path in line)
+template <bool CALL_PLAIN = true>
 __device__ __forceinline__ v2i quant8(const float* v, const Divider& d) {
-  if (__builtin_expect(d.plain, 0)) return quant8_plain(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], d.s);
+  if (__builtin_expect(d.plain, 0)) {
+    if constexpr (CALL_PLAIN) {
+      return quant8_plain(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], d.s);
+    } else {
+      const float t[8] = {v[0] / d.s, v[1] / d.s, v[2] / d.s, v[3] / d.s, v[4] / d.s, v[5] / d.s, v[6] / d.s, v[7] / d.s};
+      return pack8_fp8(t);
+    }
+  }
   float t[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) t[i] = __builtin_fmaf(v[i], d.yh, v[i] * d.yl);

@@ -109,45 +109,6 @@ struct Raw8<GLU> {
   }
 };
 
-// SwiGLU backward on load.  The loader reads a, b (unless only db is wanted) and dh; get() yields
-// eight elements of da or of db.
-struct GluBwd8 {
-  v4i a, b, d;
-  template <bool WANT_DB>
-  __device__ __forceinline__ void load(const u16* pa, uint32_t boff, int64_t gate_off, const u16* pd, uint32_t boff_d) {
-    a = ld16(pa, boff);  // a and dh are read by both teams: plain loads, kept in the caches
-    d = ld16(pd, boff_d);
-    if constexpr (!WANT_DB) b = ld16_nt(pa + gate_off, boff);
-    else b = v4i{0, 0, 0, 0};
-  }
-  __device__ __forceinline__ void zero() { a = b = d = v4i{0, 0, 0, 0}; }
-  template <bool WANT_DB>
-  __device__ __forceinline__ void get(float* v) const {
-    float fa[8], fb[8], fd[8];
-    unpack8(a, fa);
-    unpack8(b, fb);
-    unpack8(d, fd);
-#pragma unroll
-    for (int i = 0; i < 8; i += 2) {
-      float r0, r1;
-      const float rs0 = sigmoid_scaled(fa[i]), rs1 = sigmoid_scaled(fa[i + 1]);
-      if constexpr (WANT_DB) {
-        const uint32_t sl = pack_bf16x2(silu_from(fa[i], rs0), silu_from(fa[i + 1], rs1));
-        r0 = fd[i] * __uint_as_float(sl << 16);
-        r1 = fd[i + 1] * __uint_as_float(sl & 0xffff0000u);
-      } else {
-        const float sg0 = rs0 * 0x1p-16f, sg1 = rs1 * 0x1p-16f;
-        const uint32_t g = pack_bf16x2(fd[i] * fb[i], fd[i + 1] * fb[i + 1]);
-        r0 = (__uint_as_float(g << 16) * sg0) * (1.0f + fa[i] * (1.0f - sg0));
-        r1 = (__uint_as_float(g & 0xffff0000u) * sg1) * (1.0f + fa[i + 1] * (1.0f - sg1));
-      }
-      const uint32_t o = pack_bf16x2(r0, r1);
-      v[i] = __uint_as_float(o << 16);
-      v[i + 1] = __uint_as_float(o & 0xffff0000u);
-    }
-  }
-};
-
 // GELU on load (fp32 arithmetic of the torch op on a bf16 tensor, one rounding to bf16), and its
 // backward dh (cdf + x pdf) with cdf = (1 + erf(x / sqrt 2)) / 2, pdf = exp(-x^2 / 2) / sqrt(2 pi).
 template <>
@@ -267,14 +228,12 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
 constexpr int kTLd = kTile + 16;  // LDS row stride (bytes) of the transposed code tile
 // 128 rows of a tile are addressed with 32-bit byte offsets: row strides (elements, at most 4 bytes each) stay below this
 constexpr int64_t kMaxTileLd = (int64_t)1 << 22;
-// thread index inside a 256-thread tile team (a workgroup is one team, or two for the SwiGLU backward)
-__device__ __forceinline__ int team_tid() { return threadIdx.x & 255; }
 
 // `x` is the tile's origin, the same in every lane; FULL: all 128 rows are valid
 template <typename IN, bool FULL>
 __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int rows_valid,
                                           float (&v)[8][8], int64_t gate_off = 0) {
-  const int gr = team_tid() >> 4, c = team_tid() & 15;
+  const int gr = (int)threadIdx.x >> 4, c = (int)threadIdx.x & 15;
   constexpr uint32_t kEl = sizeof(typename IN::elem);
   const uint32_t off0 = ((uint32_t)(gr * 8) * ldx + (uint32_t)c * 8) * kEl;
   Raw8<IN> raw[8];
@@ -289,32 +248,13 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
   for (int i = 0; i < 8; i++) raw[i].get(v[i]);
 }
 
-// the same register tile of da (WANT_DB false) or db of one feature tile (fc1 and dh at the tile's origin)
-template <bool WANT_DB, bool FULL>
-__device__ __forceinline__ void load_tile_glu_bwd(const u16* __restrict__ fc1, uint32_t ld, int64_t gate_off,
-                                                  const u16* __restrict__ dh, uint32_t ld_dh, int rows_valid,
-                                                  float (&v)[8][8]) {
-  const int gr = team_tid() >> 4, c = team_tid() & 15;
-  const uint32_t off0 = ((uint32_t)(gr * 8) * ld + (uint32_t)c * 8) * 2, off0d = ((uint32_t)(gr * 8) * ld_dh + (uint32_t)c * 8) * 2;
-  GluBwd8 raw[8];
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    if (FULL || gr * 8 + i < rows_valid)
-      raw[i].template load<WANT_DB>(fc1, off0 + (uint32_t)i * ld * 2, gate_off, dh, off0d + (uint32_t)i * ld_dh * 2);
-    else
-      raw[i].zero();
-  }
-#pragma unroll
-  for (int i = 0; i < 8; i++) raw[i].template get<WANT_DB>(v[i]);
-}
-
 // the staged 128 x 128 code tile written as rows of 128 bytes, one 16-byte store per lane
 // (`out`: the tile's origin, the same in every lane; 128 ld_out < 2^32)
 __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t* __restrict__ out, uint32_t ld_out) {
   __syncthreads();
 #pragma unroll
   for (int n = 0; n < 4; n++) {
-    const int idx = team_tid() + 256 * n;
+    const int idx = (int)threadIdx.x + 256 * n;
     const int r = idx >> 3, ch = idx & 7;
     st_nt(out, (uint32_t)r * ld_out + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16));
   }
@@ -324,7 +264,7 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
 // out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
 __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const Divider* cdiv, uint8_t* tile_t,
                                                  uint8_t* __restrict__ out, uint32_t ld_out) {
-  const int gr = team_tid() >> 4, c = team_tid() & 15;
+  const int gr = (int)threadIdx.x >> 4, c = (int)threadIdx.x & 15;
 #pragma unroll
   for (int j = 0; j < 8; j++) {
     float col[8];
@@ -338,25 +278,18 @@ __device__ __forceinline__ void store_transposed(const float (&v)[8][8], const D
 // One 128 x 128 tile of the dual quantiser: token tile pt of group g, column tile kc.  Everything that
 // locates the tile is the same in every lane, so each access is a scalar base plus a 32-bit lane offset
 // (the launchers bound the row strides so that 128 rows stay below 2^32 bytes).
-template <typename IN, bool WANT_DB, bool FULL>
+template <typename IN, bool FULL>
 __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int nt, int64_t m0,
                                           int mvalid, int pt, int kc, uint8_t* __restrict__ q, float* __restrict__ s,
                                           uint8_t* __restrict__ q_t, float* __restrict__ s_t, uint32_t ld_t, float eps,
-                                          int64_t gate_off, u16* __restrict__ h_out, const u16* __restrict__ dh,
-                                          uint32_t ld_dh, uint8_t* tile_t, Divider* cdiv) {
+                                          int64_t gate_off, u16* __restrict__ h_out, uint8_t* tile_t, Divider* cdiv) {
   const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
   const int64_t cols = (int64_t)nt * kTile;
-  const int gr = team_tid() >> 4, c = team_tid() & 15;
+  const int gr = (int)threadIdx.x >> 4, c = (int)threadIdx.x & 15;
 
   float v[8][8];
-  if constexpr (std::is_same<IN, GLUB>::value) {
-    const int half = nt / 2;  // output column tiles [0, half) are da, [half, nt) are db
-    const int64_t f0 = (int64_t)(WANT_DB ? kc - half : kc) * kTile;
-    load_tile_glu_bwd<WANT_DB, FULL>(x + m0 * ldx + f0, ldx, gate_off, dh + m0 * ld_dh + f0, ld_dh, mvalid, v);
-  } else {
-    load_tile<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
-  }
+  load_tile<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
 
   // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
   u16* const hb = h_out ? h_out + m0 * cols + (int64_t)kc * kTile : nullptr;
@@ -388,33 +321,28 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
     part[gr][c * 8 + j] = cm[j];
   }
   __syncthreads();
-  if (team_tid() < kTile) {
-    float m = part[0][team_tid()];
+  if ((int)threadIdx.x < kTile) {
+    float m = part[0][(int)threadIdx.x];
 #pragma unroll
-    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][team_tid()]);
+    for (int i = 1; i < 16; i++) m = fmaxf(m, part[i][(int)threadIdx.x]);
     const Divider dv = make_scale(m, eps, plain_div);
-    cdiv[(team_tid() & 7) * 16 + (team_tid() >> 3)] = dv;  // [column % 8][column / 8]: lanes of a row read 16 neighbours
-    (s_t + (int64_t)pt * cols + (int64_t)kc * kTile)[team_tid()] = dv.s;
+    cdiv[((int)threadIdx.x & 7) * 16 + ((int)threadIdx.x >> 3)] = dv;  // [column % 8][column / 8]: lanes of a row read 16 neighbours
+    (s_t + (int64_t)pt * cols + (int64_t)kc * kTile)[(int)threadIdx.x] = dv.s;
   }
   __syncthreads();
   store_transposed(v, cdiv + c, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
 }
 
 template <typename IN>
-__global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void quant_dual_grouped_kernel(
+__global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
     uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
-    u16* __restrict__ h_out, const u16* __restrict__ dh = nullptr, int64_t ld_dh = 0) {
+    u16* __restrict__ h_out) {
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
-  // SwiGLU backward: two teams of 256 threads per workgroup, one for the da tile and one for the db
-  // tile of the same features, each with its own staging; both read a and dh at the same time, so
-  // the second read is served by the caches and HBM sees every input once
-  constexpr int TEAMS = std::is_same<IN, GLUB>::value ? 2 : 1;
-  const int team = TEAMS == 2 ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) : 0;
-  __shared__ __attribute__((aligned(16))) uint8_t tile_ts[TEAMS][kTile * kTLd];
-  static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_ts[0]), "the column maxima fit in the staging region");
-  __shared__ Divider cdivs[TEAMS][kTile];  // scale and divider of every column of the tile
+  __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
+  static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_t), "the column maxima fit in the staging region");
+  __shared__ Divider cdiv[kTile];  // scale and divider of every column of the tile
   __shared__ int slot;
 
   // Workgroups go to the eight XCDs in turn, and the row-wise scales of a tile are 128 single floats, one
@@ -431,32 +359,197 @@ __global__ __launch_bounds__((std::is_same<IN, GLUB>::value ? 512 : 256)) void q
       bx = (chunk - by * per_row) * 8 + (j & 7);
     }
   }
-  const int pt = (int)by;
-  int kc = (int)bx;
-  if constexpr (TEAMS == 2) kc = team * (nt / 2) + (int)bx;  // da tiles first, then db tiles
+  const int pt = (int)by, kc = (int)bx;
   const int g = __builtin_amdgcn_readfirstlane(find_group(tile_off, E, pt, &slot));
   if (g >= E) return;
   const int64_t m0 = goff[g] + (int64_t)(pt - tile_off[g]) * kTile;
   const int64_t left = goff[g + 1] - m0;
   const int mvalid = left < kTile ? (int)left : kTile;
-  uint8_t* const tile_t = tile_ts[team];
-  Divider* const cdiv = cdivs[team];
+  if (mvalid == kTile)
+    dual_tile<IN, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, gate_off, h_out, tile_t, cdiv);
+  else
+    dual_tile<IN, false>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, gate_off, h_out, tile_t, cdiv);
+}
 
-  auto run = [&](auto WANT_DB, auto FULL) {
-    dual_tile<IN, decltype(WANT_DB)::value, decltype(FULL)::value>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t,
-                                                                   (uint32_t)ld_t, eps, gate_off, h_out, dh,
-                                                                   (uint32_t)ld_dh, tile_t, cdiv);
-  };
-  auto run_full = [&](auto WANT_DB) {
-    if (mvalid == kTile) run(WANT_DB, std::true_type{});
-    else run(WANT_DB, std::false_type{});
-  };
-  if constexpr (TEAMS == 2) {
-    if (team == 0) run_full(std::false_type{});
-    else run_full(std::true_type{});
-  } else {
-    run_full(std::false_type{});
+// ---------------------------------------------------------------------------------------
+// SwiGLU backward with both quantisations: rows [a | b] plus the gradient dh of h give the [da | db] row,
+//   da = bf16(bf16(dh*b) * sig(a) * (1 + a*(1 - sig(a)))),  db = bf16(dh * bf16(silu(a))),
+// what autograd makes of the two torch ops on bf16 tensors (grouped_gemm_moe.py:331-334).  One workgroup of 512
+// threads per 128 tokens x 128 features makes the da tile and the db tile of those features from one read of a, b
+// and dh and one sigmoid per position.
+// Thread (gr = tid / 16, c = tid % 16) holds rows gr*4 .. gr*4+3, columns c*8 .. c*8+7 of both tiles.
+// ---------------------------------------------------------------------------------------
+// 4 values / one scale -> 4 codes in one dword
+__device__ __forceinline__ int quant4(const float* v, const Divider& d) {
+  float t[4];
+  if (__builtin_expect(d.plain, 0)) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) t[i] = v[i] / d.s;
+    return pack2_fp8<true>(t[2], t[3], pack2_fp8<false>(t[0], t[1], 0));
   }
+#pragma unroll
+  for (int i = 0; i < 4; i++) t[i] = __builtin_fmaf(v[i], d.yh, v[i] * d.yl);
+  return pack2_fp8<true>(t[2], t[3], pack2_fp8<false>(t[0], t[1], 0));
+}
+
+template <bool FULL>
+__device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa /* a at the tile's origin */, uint32_t ld,
+                                                     int64_t gate_off, const u16* __restrict__ xd, uint32_t ld_dh, int nt,
+                                                     int64_t m0, int mvalid, int pt, int f, uint8_t* __restrict__ q,
+                                                     float* __restrict__ s, uint8_t* __restrict__ q_t,
+                                                     float* __restrict__ s_t, uint32_t ld_t, u16* __restrict__ g_out,
+                                                     uint8_t (*tile_t)[kTile * kTLd], Divider (*cdiv)[kTile]) {
+  const int tid = threadIdx.x, gr = tid >> 4, c = tid & 15;
+  const int half = nt / 2;
+  const int64_t cols = (int64_t)nt * kTile;
+  const uint32_t ucols = (uint32_t)cols;
+  // ---- loads, then da and db of the thread's 4 x 8 positions
+  v4i ra[4], rb[4], rd[4];
+  {
+    const uint32_t off0 = ((uint32_t)(gr * 4) * ld + (uint32_t)c * 8) * 2, off0d = ((uint32_t)(gr * 4) * ld_dh + (uint32_t)c * 8) * 2;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      if (FULL || gr * 4 + i < mvalid) {
+        ra[i] = ld16_nt(xa, off0 + (uint32_t)i * ld * 2);
+        rb[i] = ld16_nt(xa + gate_off, off0 + (uint32_t)i * ld * 2);
+        rd[i] = ld16_nt(xd, off0d + (uint32_t)i * ld_dh * 2);
+      } else {
+        ra[i] = rb[i] = rd[i] = v4i{0, 0, 0, 0};
+      }
+    }
+  }
+  uint32_t vp[2][4][4];  // [da | db][row][column pair]: the results are bf16 numbers and wait for the column pass packed
+  float (*part)[32][kTile] = reinterpret_cast<float (*)[32][kTile]>(&tile_t[0][0]);  // [2][32][128] floats: dead before the staging
+  static_assert(sizeof(float) * 2 * 32 * kTile <= 2 * sizeof(tile_t[0]), "the column maxima fit in the staging regions");
+  float cm[2][8];
+#pragma unroll
+  for (int w = 0; w < 2; w++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) cm[w][j] = 0.f;
+  // one row at a time, from the packed inputs to the stored codes of both tiles
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    float fa[8], fb[8], fd[8], v[2][8];
+    unpack8(ra[i], fa);
+    unpack8(rb[i], fb);
+    unpack8(rd[i], fd);
+#pragma unroll
+    for (int k = 0; k < 8; k += 2) {
+      const float rs0 = sigmoid_scaled(fa[k]), rs1 = sigmoid_scaled(fa[k + 1]);
+      // db = bf16(dh * bf16(silu(a)))
+      const uint32_t sl = pack_bf16x2(silu_from(fa[k], rs0), silu_from(fa[k + 1], rs1));
+      const uint32_t ob = pack_bf16x2(fd[k] * __uint_as_float(sl << 16), fd[k + 1] * __uint_as_float(sl & 0xffff0000u));
+      vp[1][i][k / 2] = ob;
+      v[1][k] = __uint_as_float(ob << 16);
+      v[1][k + 1] = __uint_as_float(ob & 0xffff0000u);
+      // da = bf16(bf16(dh * b) * sig(a) * (1 + a * (1 - sig(a))))
+      const float sg0 = rs0 * 0x1p-16f, sg1 = rs1 * 0x1p-16f;
+      const uint32_t gb = pack_bf16x2(fd[k] * fb[k], fd[k + 1] * fb[k + 1]);
+      const uint32_t oa = pack_bf16x2((__uint_as_float(gb << 16) * sg0) * (1.0f + fa[k] * (1.0f - sg0)),
+                                      (__uint_as_float(gb & 0xffff0000u) * sg1) * (1.0f + fa[k + 1] * (1.0f - sg1)));
+      vp[0][i][k / 2] = oa;
+      v[0][k] = __uint_as_float(oa << 16);
+      v[0][k + 1] = __uint_as_float(oa & 0xffff0000u);
+    }
+    const uint32_t r = (uint32_t)(gr * 4 + i);
+    const bool live = FULL || (int)r < mvalid;
+#pragma unroll
+    for (int w = 0; w < 2; w++) {
+      const int kc = w == 0 ? f : half + f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) cm[w][j] = fmaxf(cm[w][j], fabsf(v[w][j]));
+      if (g_out != nullptr && live)
+        st_nt(g_out + m0 * cols + (int64_t)kc * kTile, (r * ucols + (uint32_t)c * 8) * 2,
+              v4i{(int)vp[w][i][0], (int)vp[w][i][1], (int)vp[w][i][2], (int)vp[w][i][3]});
+      if (q != nullptr) {
+        const Divider dv = make_scale(row16_max(amax8(v[w])), 0.f, false);
+        const v2i codes = quant8<false>(v[w], dv);
+        if (live) {
+          st_nt(q + m0 * cols + (int64_t)kc * kTile, r * ucols + (uint32_t)c * 8, codes);
+          if (c == 0) *reinterpret_cast<float*>(reinterpret_cast<char*>(s + m0 * nt + kc) + r * (uint32_t)nt * 4) = dv.s;
+        }
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < 2; w++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) asm volatile("" : "+v"(vp[w][i][j]));  // the row is finished before the next one starts
+  }
+#pragma unroll
+  for (int w = 0; w < 2; w++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) part[w][gr][c * 8 + j] = cm[w][j];
+  __syncthreads();
+  if (tid < 2 * kTile) {
+    const int w = tid >> 7, col = tid & (kTile - 1);
+    float m = part[w][0][col];
+#pragma unroll
+    for (int i = 1; i < 32; i++) m = fmaxf(m, part[w][i][col]);
+    const Divider dv = make_scale(m, 0.f, false);
+    cdiv[w][(col & 7) * 16 + (col >> 3)] = dv;  // [column % 8][column / 8]: lanes of a row read 16 neighbours
+    (s_t + (int64_t)pt * cols + (int64_t)(w == 0 ? f : half + f) * kTile)[col] = dv.s;
+  }
+  __syncthreads();
+  // ---- transposed codes through the LDS
+#pragma unroll
+  for (int w = 0; w < 2; w++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      float col[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) col[i] = __uint_as_float(j & 1 ? vp[w][i][j / 2] & 0xffff0000u : vp[w][i][j / 2] << 16);
+      *reinterpret_cast<int*>(&tile_t[w][(c * 8 + j) * kTLd + gr * 4]) = quant4(col, cdiv[w][j * 16 + c]);
+      if (j % 4 == 3) __builtin_amdgcn_sched_barrier(0);  // a few dividers at a time: sixteen of them are 64 registers
+    }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < 2; w++) {
+    uint8_t* const out = q_t + (int64_t)(w == 0 ? f : half + f) * kTile * ld_t + (int64_t)pt * kTile;
+#pragma unroll
+    for (int n = 0; n < 2; n++) {
+      const int idx = tid + 512 * n;
+      const int r = idx >> 3, ch = idx & 7;
+      st_nt(out, (uint32_t)r * ld_t + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(&tile_t[w][r * kTLd + ch * 16]));
+    }
+  }
+}
+
+__global__ __launch_bounds__(512, 4) void swiglu_bwd_dual_kernel(const u16* __restrict__ fc1, int64_t ld, int64_t gate_off,
+                                                              const u16* __restrict__ dh, int64_t ld_dh, int nt,
+                                                              const int64_t* __restrict__ goff,
+                                                              const int32_t* __restrict__ tile_off, int E,
+                                                              uint8_t* __restrict__ q, float* __restrict__ s,
+                                                              uint8_t* __restrict__ q_t, float* __restrict__ s_t,
+                                                              int64_t ld_t, u16* __restrict__ g_out) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile_ts[2][kTile * kTLd];
+  __shared__ Divider cdivs[2][kTile];
+  __shared__ int slot;
+  // consecutive workgroups of one XCD take the eight consecutive feature tiles of a scale sector
+  // (see quant_dual_grouped_kernel)
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  {
+    const uint32_t ntx = gridDim.x, per_row = ntx >> 3;
+    const uint32_t lin = by * ntx + bx, chunks = gridDim.y * per_row;
+    if ((ntx & 7) == 0 && lin < (chunks & ~7u) * 8) {
+      const uint32_t j = lin >> 3, chunk = (j & ~7u) + (lin & 7);
+      by = chunk / per_row;
+      bx = (chunk - by * per_row) * 8 + (j & 7);
+    }
+  }
+  const int pt = (int)by, f = (int)bx;
+  const int g = __builtin_amdgcn_readfirstlane(find_group(tile_off, E, pt, &slot));
+  if (g >= E) return;
+  const int64_t m0 = goff[g] + (int64_t)(pt - tile_off[g]) * kTile;
+  const int64_t left = goff[g + 1] - m0;
+  const int mvalid = left < kTile ? (int)left : kTile;
+  const u16* const xa = fc1 + m0 * ld + (int64_t)f * kTile;
+  const u16* const xd = dh + m0 * ld_dh + (int64_t)f * kTile;
+  if (mvalid == kTile)
+    swiglu_bwd_dual_tile<true>(xa, (uint32_t)ld, gate_off, xd, (uint32_t)ld_dh, nt, m0, mvalid, pt, f, q, s, q_t, s_t,
+                               (uint32_t)ld_t, g_out, tile_ts, cdivs);
+  else
+    swiglu_bwd_dual_tile<false>(xa, (uint32_t)ld, gate_off, xd, (uint32_t)ld_dh, nt, m0, mvalid, pt, f, q, s, q_t, s_t,
+                                (uint32_t)ld_t, g_out, tile_ts, cdivs);
 }
 
 // The 8x8 byte matrix held as eight rows of two dwords, transposed with byte permutes: cols[j]
@@ -816,8 +909,8 @@ extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t 
   if (rc) return rc;
   const int nt = (int)(2 * F / kTile);
   dim3 grid((unsigned)(nt / 2), (unsigned)grid_tiles), block(512);  // two teams: the da and the db tile of a feature tile
-  quant_dual_grouped_kernel<GLUB><<<grid, block, 0, st>>>((const u16*)fc1, ld, nt, group_offsets, tile_ws, E, q, s, q_t, s_t,
-                                                          ld_t, 0.f, F, (u16*)g_out, (const u16*)dh, ld_dh);
+  swiglu_bwd_dual_kernel<<<grid, block, 0, st>>>((const u16*)fc1, ld, F, (const u16*)dh, ld_dh, nt, group_offsets, tile_ws, E,
+                                                 q, s, q_t, s_t, ld_t, (u16*)g_out);
   AAMD_LAUNCH_CHECK("swiglu_bwd_quant_dual_grouped");
   return AAMD_OK;
 }
