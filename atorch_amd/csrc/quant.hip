@@ -34,6 +34,7 @@ struct Raw8<BF16> {
   v4i a;
   __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t) { a = ld16_nt(p, boff); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a)); }
   __device__ __forceinline__ void get(float* v) const { unpack8(a, v); }
 };
 template <>
@@ -44,6 +45,7 @@ struct Raw8<F32> {
     b = ld16_nt(p + 4, boff);
   }
   __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a), "+v"(b)); }
   __device__ __forceinline__ void get(float* v) const {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -58,6 +60,7 @@ struct Raw8<F16> {
   v4i a;
   __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t) { a = ld16_nt(p, boff); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a)); }
   __device__ __forceinline__ void get(float* v) const {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -93,6 +96,7 @@ struct Raw8<GLU> {
     b = ld16_nt(p + gate_off, boff);
   }
   __device__ __forceinline__ void zero() { a = b = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a), "+v"(b)); }
   __device__ __forceinline__ void get(float* v) const {
     float fa[8], fb[8];
     unpack8(a, fa);
@@ -116,6 +120,7 @@ struct Raw8<GELU> {
   v4i a;
   __device__ __forceinline__ void load(const u16* p, uint32_t boff, int64_t) { a = ld16_nt(p, boff); }
   __device__ __forceinline__ void zero() { a = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a)); }
   __device__ __forceinline__ void get(float* v) const {
     float x[8];
     unpack8(a, x);
@@ -137,6 +142,7 @@ struct Raw8<GELUB> {
     d = ld16_nt(p + dh_off, boff);
   }
   __device__ __forceinline__ void zero() { a = d = v4i{0, 0, 0, 0}; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a), "+v"(d)); }
   __device__ __forceinline__ void get(float* v) const {
     float x[8], g[8];
     unpack8(a, x);
@@ -231,12 +237,11 @@ constexpr int64_t kMaxTileLd = (int64_t)1 << 22;
 
 // `x` is the tile's origin, the same in every lane; FULL: all 128 rows are valid
 template <typename IN, bool FULL>
-__device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int rows_valid,
-                                          float (&v)[8][8], int64_t gate_off = 0) {
+__device__ __forceinline__ void issue_tile_loads(const typename IN::elem* __restrict__ x, uint32_t ldx, int rows_valid,
+                                                 Raw8<IN> (&raw)[8], int64_t gate_off = 0) {
   const int gr = (int)threadIdx.x >> 4, c = (int)threadIdx.x & 15;
   constexpr uint32_t kEl = sizeof(typename IN::elem);
   const uint32_t off0 = ((uint32_t)(gr * 8) * ldx + (uint32_t)c * 8) * kEl;
-  Raw8<IN> raw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     if (FULL || gr * 8 + i < rows_valid)
@@ -244,6 +249,12 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
     else
       raw[i].zero();
   }
+}
+template <typename IN, bool FULL>
+__device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int rows_valid,
+                                          float (&v)[8][8], int64_t gate_off = 0) {
+  Raw8<IN> raw[8];
+  issue_tile_loads<IN, FULL>(x, ldx, rows_valid, raw, gate_off);
 #pragma unroll
   for (int i = 0; i < 8; i++) raw[i].get(v[i]);
 }
@@ -260,21 +271,6 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
   }
 }
 
-// codes of the 8x8 register block, transposed through LDS, written as rows of 128 bytes:
-// out[(col) * ld_out + token], one 16-byte store per lane, 8 lanes per row.
-__device__ __forceinline__ void store_transposed(const float (&v)[8][8], const Divider* cdiv, uint8_t* tile_t,
-                                                 uint8_t* __restrict__ out, uint32_t ld_out) {
-  const int gr = (int)threadIdx.x >> 4, c = (int)threadIdx.x & 15;
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    float col[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) col[i] = v[i][j];
-    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cdiv[j * 16]);
-  }
-  store_staged_tile(tile_t, out, ld_out);
-}
-
 // One 128 x 128 tile of the dual quantiser: token tile pt of group g, column tile kc.  Everything that
 // locates the tile is the same in every lane, so each access is a scalar base plus a 32-bit lane offset
 // (the launchers bound the row strides so that 128 rows stay below 2^32 bytes).
@@ -288,8 +284,14 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
   const int64_t cols = (int64_t)nt * kTile;
   const int gr = (int)threadIdx.x >> 4, c = (int)threadIdx.x & 15;
 
-  float v[8][8];
-  load_tile<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, v, gate_off);
+  // The GELU kernels hold their results, which are bf16 numbers, packed two to a register until the column pass
+  // (the erf evaluation needs the registers: unpacked, two workgroups fit on a CU instead of four).  For the other
+  // inputs the 64 values of a thread stay in fp32: packed they measured no faster.
+  constexpr bool kPacked = std::is_same<IN, GELU>::value || std::is_same<IN, GELUB>::value;
+  Raw8<IN> raw[8];
+  issue_tile_loads<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, raw, gate_off);
+  float v[kPacked ? 1 : 8][8];
+  uint32_t vp[kPacked ? 8 : 1][4];
 
   // row-wise 1x128 codes and scales (a tile row lives in one 16-lane DPP row)
   u16* const hb = h_out ? h_out + m0 * cols + (int64_t)kc * kTile : nullptr;
@@ -303,21 +305,40 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
   for (int i = 0; i < 8; i++) {
     const uint32_t r = (uint32_t)(gr * 8 + i);
     const bool live = FULL || (int)r < mvalid;
-    if (hb != nullptr && live) st_nt(hb, (r * ucols + (uint32_t)c * 8) * 2, pack8_bf16(v[i]));
+    float (&vi)[8] = v[kPacked ? 0 : i];
+    // (a row is unpacked where its turn comes: hoisted to the top, the rows of the whole tile would be live unpacked)
+    if constexpr (kPacked) raw[i].pin();
+    raw[i].get(vi);
+    if constexpr (kPacked) {
+      v4i pk;
+      if constexpr (std::is_same<IN, BF16>::value) pk = raw[i].a;  // the input is the packed row
+      else pk = pack8_bf16(vi);
+#pragma unroll
+      for (int k = 0; k < 4; k++) vp[i][k] = (uint32_t)pk[k];
+#pragma unroll
+      for (int j = 0; j < 8; j++) cm[j] = fmaxf(cm[j], fabsf(vi[j]));
+    }
+    if (hb != nullptr && live) st_nt(hb, (r * ucols + (uint32_t)c * 8) * 2, pack8_bf16(vi));
     if (qb != nullptr) {
-      const Divider dv = make_scale(row16_max(amax8(v[i])), eps, plain_div);
-      const v2i codes = quant8(v[i], dv);
+      const Divider dv = make_scale(row16_max(amax8(vi)), eps, plain_div);
+      const v2i codes = quant8(vi, dv);
       if (live) {
         st_nt(qb, r * ucols + (uint32_t)c * 8, codes);
         if (c == 0) *reinterpret_cast<float*>(reinterpret_cast<char*>(sb) + r * (uint32_t)nt * 4) = dv.s;
       }
     }
+    if constexpr (kPacked) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) asm volatile("" : "+v"(vp[i][k]));  // the row is finished before the next one is unpacked
+    }
   }
   // column amax over the 128 tokens of the tile (two rows per three-operand maximum)
 #pragma unroll
   for (int j = 0; j < 8; j++) {
+    if constexpr (!kPacked) {
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) cm[j] = fmaxf(fmaxf(cm[j], fabsf(v[i][j])), fabsf(v[i + 1][j]));
+      for (int i = 0; i < 8; i += 2) cm[j] = fmaxf(fmaxf(cm[j], fabsf(v[i][j])), fabsf(v[i + 1][j]));
+    }
     part[gr][c * 8 + j] = cm[j];
   }
   __syncthreads();
@@ -330,7 +351,18 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
     (s_t + (int64_t)pt * cols + (int64_t)kc * kTile)[(int)threadIdx.x] = dv.s;
   }
   __syncthreads();
-  store_transposed(v, cdiv + c, tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
+  // codes of the 8x8 register block, transposed through LDS, written as rows of 128 bytes
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    float col[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if constexpr (kPacked) col[i] = __uint_as_float(j & 1 ? vp[i][j / 2] & 0xffff0000u : vp[i][j / 2] << 16);
+      else col[i] = v[i][j];
+    }
+    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cdiv[j * 16 + c]);
+  }
+  store_staged_tile(tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
 }
 
 template <typename IN>
