@@ -650,22 +650,43 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
     // Scales of this pipeline come in batches of eight contraction blocks only (the launcher takes the other
-    // configuration when K has fewer than eight blocks or the scale rows are not 16-byte aligned), so a
+    // configuration when K has fewer than eight blocks), so a
     // step issues no scale load and takes no branch: batch b (blocks 8 b .. 8 b + 7, the last one shifted
     // back to end at the last block) is requested behind barrier P of step 8 (b - 1), eight steps before
     // its first use.  L scales: every wave fetches 32 rows x 32 bytes into LsB[b & 1][row][8]; R block
     // scales: wave 0 fetches the tile's two 128-row blocks x 32 bytes into RsB[b & 1][block][8] (lanes past
     // the fourth repeat those addresses: the direct-to-LDS load always writes 1 KB).
+    // Scale rows that are not 16-byte aligned (a number of contraction blocks that is not a multiple of four, an
+    // unaligned base) take 4-byte loads instead: four per wave and batch for the L scales (lane l of load q fetches
+    // float 64 q + l of the wave's 32 rows x 8 floats), one for the R scales.
     float* const RsB0 = Sc0;  // [2][NT] floats, the first 16 of each in use
+    const bool x4 = p.ls_batch == 1;
     const int rblocks = rvalid / kTile;
     const int rlane_blk = ((lane >> 1) & 1) < rblocks ? (lane >> 1) & 1 : rblocks - 1;
     const uint32_t roff = ((uint32_t)rlane_blk * (uint32_t)p.rs_row_stride + (uint32_t)(lane & 1) * 4u) * 4u;
+    const int rlane_blk1 = ((lane >> 3) & 1) < rblocks ? (lane >> 3) & 1 : rblocks - 1;
+    const uint32_t roff1 = ((uint32_t)rlane_blk1 * (uint32_t)p.rs_row_stride + (uint32_t)(lane & 7)) * 4u;
+    uint32_t boff1[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int row = wave * 32 + q * 8 + (lane >> 3);
+      boff1[q] = ((uint32_t)(row < lvalid ? row : lvalid - 1) * (uint32_t)p.ls_row_stride + (uint32_t)(lane & 7)) * 4u;
+    }
     auto dma_batches = [&](int b) {
-      dma_scale_batch(b);
-      if (wave == 0) {
-        const uint8_t* sb = reinterpret_cast<const uint8_t*>(Rsg + uniform_i64((r0 / kTile) * p.rs_row_stride + batch_start(b)));
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     ::"v"(roff), "s"(sb), "s"(lds_addr(RsB0 + (b & 1) * NT)) : "memory");
+      const uint8_t* lsb = reinterpret_cast<const uint8_t*>(Lsg + uniform_i64(l0 * p.ls_row_stride + batch_start(b)));
+      const uint8_t* rsb = reinterpret_cast<const uint8_t*>(Rsg + uniform_i64((r0 / kTile) * p.rs_row_stride + batch_start(b)));
+      const uint32_t ldst = lds_addr(LsB0 + (b & 1) * (BM * 8)) + (uint32_t)(wave * 1024);
+      const uint32_t rdst = lds_addr(RsB0 + (b & 1) * NT);
+      if (x4) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(boff), "s"(lsb), "s"(ldst) : "memory");
+        if (wave == 0)
+          asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(roff), "s"(rsb), "s"(rdst) : "memory");
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(boff1[q]), "s"(lsb), "s"(ldst + (uint32_t)(q * 256)) : "memory");
+        if (wave == 0)
+          asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(roff1), "s"(rsb), "s"(rdst) : "memory");
       }
     };
     if (nkb > 0) {
@@ -765,18 +786,20 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #pragma unroll
           for (int j = 0; j < C::WTL; j++) cs[j] = csn[j] * rblkn;
         };
-        // runs of eight steps (the contraction has a multiple of four blocks, at least eight), two steps per
-        // trip so that the stage addresses are compile-time constants
+        // runs of eight steps (the contraction has at least eight blocks; the last run may be shorter), two
+        // steps per trip so that the stage addresses are compile-time constants
         constexpr std::integral_constant<int, 0> S0{};
         constexpr std::integral_constant<int, 1> S1{};
         for (int kb = 0; kb < nkb; kb += 8) {
           const int n = nkb - kb < 8 ? nkb - kb : 8;
           step(kb, S0, std::true_type{});
-          step(kb + 1, S1, std::false_type{});
-          for (int kk = 2; kk < n; kk += 2) {
+          if (n > 1) step(kb + 1, S1, std::false_type{});
+          int kk = 2;
+          for (; kk + 1 < n; kk += 2) {
             step(kb + kk, S0, std::false_type{});
             step(kb + kk + 1, S1, std::false_type{});
           }
+          if (kk < n) step(kb + kk, S0, std::false_type{});  // odd number of steps
         }
         __builtin_amdgcn_sched_barrier(0);
         fold(C::WTR - 1, C::WTL - 1, cs_last);
@@ -792,10 +815,12 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 #pragma unroll
           for (int n = 0; n < C::RCH; n++) dmaR_tile(n, k2, Rc);
         };
-        for (int kb = 0; kb < nkb; kb += 2) {
+        int kb = 0;
+        for (; kb + 1 < nkb; kb += 2) {
           step(kb, Lbuf0, Rbuf0, (kb & 7) == 0);
           step(kb + 1, Lbuf1, Rbuf1, false);
         }
+        if (kb < nkb) step(kb, Lbuf0, Rbuf0, (kb & 7) == 0);
       }
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the trailing loads must not land in the epilogue's staging
     }
@@ -1016,12 +1041,13 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   AAMD_REQUIRE(K > 0, "grouped_gemm_nt: K must be positive");
   AAMD_REQUIRE(lda < (1LL << 23) && K < (1LL << 23), "grouped_gemm_nt: row stride too large");
   hipStream_t st = (hipStream_t)stream;
-  // 16-byte loads of scale batches need aligned rows and whole groups of four blocks
-  const bool batches = (K / kBK) >= 8 && (K / kBK) % 4 == 0 && aligned16(a_s) && g_opt.ls_batch != 0;
+  // scale batches of eight contraction blocks; their 16-byte loads need aligned rows and whole groups of four blocks
+  const bool batches = (K / kBK) >= 8 && g_opt.ls_batch != 0;
+  const bool batches16 = batches && (K / kBK) % 4 == 0 && aligned16(a_s);
   // tile-scaled B carries per-row R scales: use the configuration that has room for them; the 256x256
-  // configuration takes all its scales in batches
+  // configuration takes all its scales in batches (with 4-byte loads where the rows are not aligned)
   const bool large = use_large_tiles(((M + 255) / 256 + (group_offsets ? E : 0)) * ((N + 255) / 256), true) &&
-                     (b_tile_scaled || (batches && aligned16(b_s)));
+                     (b_tile_scaled || batches);
   const int BM = large ? CfgLarge::BM : CfgSmall::BM;
   const int BN = large ? (b_tile_scaled ? CfgWgrad::BN : CfgLarge::BN) : CfgSmall::BN;
   if (group_offsets) {
@@ -1030,7 +1056,8 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   }
   GemmParams p = {};
   p.L = a; p.ldl = lda; p.Ls = a_s; p.ls_row_stride = K / kBK; p.ls_blk_stride = 1;
-  p.ls_batch = batches;
+  // 1: batches by 16-byte loads; 2 (256x256 configuration only): by 4-byte loads
+  p.ls_batch = large && !b_tile_scaled ? (batches16 && aligned16(b_s) ? 1 : 2) : (batches16 ? 1 : 0);
   p.R = b; p.ldr = K; p.r_group_stride = N * K;
   p.Rs = b_s;
   p.rs_row_stride = K / kBK; p.rs_blk_stride = 1;

@@ -37,7 +37,7 @@ TILE = 128
 # this file (with --copy-probe: a plain 1 GiB copy reads FETCH_SIZE*2.0 KiB, WRITE_SIZE*1.0 KiB), averaged
 # over that kernel's launches of one step.  Counters cannot be read from inside the process, so the
 # figures are recorded here beside the profile summaries they come from (profiles/*.txt).
-MEASURED_TRAFFIC_BYTES = {"c2": 7.18e9, "c5": 4.830e9}
+MEASURED_TRAFFIC_BYTES = {"c2": 7.13e9, "c5": 4.830e9}
 
 
 def parse():

@@ -496,14 +496,15 @@ def test_fp8_gemm_tile_scaled_b_large_tiles(dev, out_dtype):
     assert torch.equal(c, c_small)
 
 
-@pytest.mark.parametrize("K", [512, 1024, 1536, 2560, 1152], ids=lambda k: f"K{k}")
+@pytest.mark.parametrize("K", [512, 1024, 1536, 2560, 1152, 1408, 2816], ids=lambda k: f"K{k}")
 def test_grouped_gemm_nt_scale_batches_of_the_large_tiles(dev, K):
     """The 256x256 configuration takes its scales in batches of eight contraction blocks: exactly one
-    batch (K = 1024), a last batch shifted back to end at the last block (1536, 2560), and contractions
-    that cannot be batched (512: fewer than eight blocks; 1152: not a multiple of four blocks), which the
-    launcher gives to the 128x128 configuration.  Ragged groups with an empty one, a partial last R tile
-    (N = 640), bias; against the float64 definition on the device and, bit for bit, against the pinned
-    128x128 configuration, which adds the same products in the same order."""
+    batch (K = 1024), a last batch shifted back to end at the last block (1536, 2560), scale rows that are
+    not 16-byte aligned and take 4-byte loads, with an odd number of steps (1152, 1408) and an even one
+    (2816), and a contraction with fewer than eight blocks (512), which the launcher gives to the 128x128
+    configuration.  Ragged groups with an empty one, a partial last R tile (N = 640), bias; against the
+    float64 definition on the device and, bit for bit, against the pinned 128x128 configuration, which adds
+    the same products in the same order."""
     from atorch_amd import kernels
 
     E, N = 4, 640
