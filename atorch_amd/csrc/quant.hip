@@ -286,7 +286,7 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
 
   // The GELU kernels hold their results, which are bf16 numbers, packed two to a register until the column pass
   // (the erf evaluation needs the registers: unpacked, two workgroups fit on a CU instead of four).  For the other
-  // inputs the 64 values of a thread stay in fp32: packed they measured no faster.
+  // inputs the 64 values of a thread stay in fp32: the packed form compiles to more registers there, not fewer.
   constexpr bool kPacked = std::is_same<IN, GELU>::value || std::is_same<IN, GELUB>::value;
   Raw8<IN> raw[8];
   issue_tile_loads<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, raw, gate_off);
