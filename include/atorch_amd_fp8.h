@@ -220,8 +220,9 @@ int aamd_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uin
  * Pins a launch choice of the grouped GEMMs that the library otherwise makes by itself (for tests
  * and tuning runs; no counterpart in the reference).  value -1 restores the library's choice.
  *   "tile": 0 = 128x128 tiles, 1 = the large configuration; "group_r": tile order groups R tiles (1)
- *   or L tiles (0); "gl": tiles sharing a panel in the tile order; "ls_batch": 0 = activation scales
- *   fetched one contraction block at a time.  Process-wide; not synchronised with running launches.
+ *   or L tiles (0); "gl": tiles sharing a panel in the tile order; "ls_batch": 0 = scales fetched one
+ *   contraction block at a time (which the 128x128 tiles do: the large configuration of the block-scaled GEMM takes
+ *   its scales in batches only and is then not chosen).  Process-wide; not synchronised with running launches.
  */
 int aamd_gemm_set_option(const char *name, int value);
 
