@@ -357,11 +357,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // All loads of the contraction loop are issued from inline assembly, with the wait counts kept
   // by hand: the compiler's own bookkeeping of direct-to-LDS loads is conservative (it tracks
   // eight of them individually and otherwise waits for every outstanding load).  Per step and
-  // thread: LCH + RCH 16-byte tile loads and one 4-byte scale load; all of them write LDS only,
+  // thread: LCH + RCH 16-byte tile loads and the scale loads; all of them write LDS only,
   // so no VGPR is ever written behind the compiler's back.
   auto lds_addr = [](const void* q) { return (uint32_t)(uintptr_t)(lds_ptr_t)q; };
   const uint32_t soff_b = soff * 4u;
-  constexpr int kScaleLd = 1;
   // L scales of a row-major [rows, K/128] operand: one 4-byte value per row and step would touch
   // as many cache lines as the tile itself.  Instead 32 bytes per row (eight contraction blocks)
   // are fetched every eighth step, 16 bytes per thread, into [row][8] floats.  The last batch is

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(512) void unpermute_combine_kernel(const typename Y
   __shared__ int srow[kMaxTopk];
   __shared__ float sprob[kMaxTopk];
   const int64_t t = blockIdx.x;
-  if (threadIdx.x < topk) {
+  if ((int)threadIdx.x < topk) {
     int r = row_map[t * topk + threadIdx.x];
     if (r >= M) r = -1;
     srow[threadIdx.x] = r;
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(256) void route_rowscan_kernel(int32_t* __restrict_
     buf[threadIdx.x] = v;
     __syncthreads();
     for (int d = 1; d < 256; d <<= 1) {
-      const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+      const int t = (int)threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
       __syncthreads();
       buf[threadIdx.x] += t;
       __syncthreads();
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(256) void route_goff_kernel(const int32_t* __restri
     buf[threadIdx.x] = e < E ? totals[e] : 0;
     __syncthreads();
     for (int d = 1; d < 256; d <<= 1) {
-      const int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+      const int t = (int)threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
       __syncthreads();
       buf[threadIdx.x] += t;
       __syncthreads();
@@ -424,10 +424,10 @@ __global__ __launch_bounds__(256) void fill_zero_f32_kernel(float* __restrict__ 
 // grouped by expert cost one set of atomics per workgroup and expert.
 constexpr int kBgRows = 128;
 template <typename ID>
-__global__ __launch_bounds__(256) void bias_gather_bgrad_kernel(const v4i* __restrict__ grad, const ID* __restrict__ bin_ids,
+__global__ __launch_bounds__(512) void bias_gather_bgrad_kernel(const v4i* __restrict__ grad, const ID* __restrict__ bin_ids,
                                                                 int64_t T, int row_chunks, int E, bool is_bf16,
                                                                 float* __restrict__ bgrad) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= row_chunks) return;
   const int64_t t0 = (int64_t)blockIdx.y * kBgRows;
   const int64_t t1 = t0 + kBgRows < T ? t0 + kBgRows : T;
@@ -478,6 +478,19 @@ __global__ __launch_bounds__(256) void bias_gather_bgrad_kernel(const v4i* __res
 
 using namespace aamd;
 
+// Workgroup size for kernels that walk a row in 16-byte chunks, one chunk per lane and trip: 256 lanes unless
+// another multiple of 64 leaves fewer lanes idle in the last trip (7168 columns of bf16 are 896 chunks: 448 lanes
+// make two full trips, 256 would leave the fourth half empty).
+static int threads_for_row_chunks(int64_t chunks) {
+  int threads = 256;
+  int64_t waste = (chunks + 255) / 256 * 256 - chunks;
+  for (int b = 512; b >= 128; b -= 64) {
+    const int64_t w = (chunks + b - 1) / b * b - chunks;
+    if (w < waste) { waste = w; threads = b; }
+  }
+  return threads;
+}
+
 extern "C" int aamd_bias_gather_add(const void* inp, const void* bias, const void* bin_ids, int ids_are_i64, int64_t T,
                                     int64_t H, int E, int dtype, void* out, void* stream) {
   AAMD_REQUIRE(dtype == AAMD_BF16 || dtype == AAMD_F32, "bias_gather_add: unsupported dtype %d", dtype);
@@ -519,7 +532,8 @@ extern "C" int aamd_bias_gather_add_bgrad(const void* grad, const void* bin_ids,
   AAMD_REQUIRE(((uintptr_t)grad & 15) == 0, "bias_gather_add_bgrad: grad must be 16-byte aligned");
   const int64_t rc = row_bytes / 16, row_blocks = (T + kBgRows - 1) / kBgRows;
   AAMD_REQUIRE(rc < 0x7fffffffLL && row_blocks <= 65535, "bias_gather_add_bgrad: more than 65535 * 128 rows");
-  dim3 grid((unsigned)((rc + 255) / 256), (unsigned)row_blocks), block(256);
+  const int threads = threads_for_row_chunks(rc);
+  dim3 grid((unsigned)((rc + threads - 1) / threads), (unsigned)row_blocks), block((unsigned)threads);
   if (ids_are_i64)
     bias_gather_bgrad_kernel<int64_t><<<grid, block, 0, st>>>((const v4i*)grad, (const int64_t*)bin_ids, T, (int)rc, E,
                                                               dtype == AAMD_BF16, bgrad);
@@ -545,15 +559,8 @@ extern "C" int aamd_unpermute_combine(const void* y, int y_dtype, int64_t M, int
   AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs != nullptr, "unpermute_combine: probs missing");
   AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0, "unpermute_combine: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  // one workgroup per token, one 16-byte chunk of the row per lane and trip: the workgroup size that
-  // leaves the fewest lanes idle in the last trip (7168 columns of bf16: 448 lanes, two full trips)
-  const int64_t chunks = H / (y_dtype == AAMD_BF16 ? 8 : 4);
-  int threads = 256;
-  int64_t waste = (chunks + 255) / 256 * 256 - chunks;
-  for (int b = 512; b >= 128; b -= 64) {
-    const int64_t w = (chunks + b - 1) / b * b - chunks;
-    if (w < waste) { waste = w; threads = b; }
-  }
+  // one workgroup per token, one 16-byte chunk of the row per lane and trip
+  const int threads = threads_for_row_chunks(H / (y_dtype == AAMD_BF16 ? 8 : 4));
   dim3 grid((unsigned)T), block((unsigned)threads);
   if (y_dtype == AAMD_BF16) {
     const int H8 = (int)(H / 8);

@@ -668,7 +668,7 @@ __global__ __launch_bounds__(256) void group_tile_offsets_kernel(const int64_t* 
     buf[threadIdx.x] = n;
     __syncthreads();
     for (int d = 1; d < 256; d <<= 1) {
-      int t = threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
+      int t = (int)threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
       __syncthreads();
       buf[threadIdx.x] += t;
       __syncthreads();
