@@ -324,7 +324,7 @@ def test_permute_quant_commutes(oracle, dev, T, E, k, H):
 # a10: unpermute + combine
 # ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("probs_dtype", [torch.bfloat16, torch.float32, None])
-@pytest.mark.parametrize("T,E,k,H", [(256, 8, 2, 512), (100, 64, 8, 1024)])
+@pytest.mark.parametrize("T,E,k,H", [(256, 8, 2, 512), (100, 64, 8, 1024), (37, 8, 2, 7168), (64, 4, 3, 5120)])
 def test_unpermute_combine(oracle, dev, probs_dtype, T, E, k, H):
     from atorch_amd.token_dispatcher import unpermute
 
@@ -690,7 +690,7 @@ def test_unpermute_matches_torch_ops_on_the_gpu(dev):
 # ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("ids_dtype", [torch.int64, torch.int32])
-@pytest.mark.parametrize("T,H,E", [(1, 8, 1), (300, 136, 5), (4097, 1024, 64)])
+@pytest.mark.parametrize("T,H,E", [(1, 8, 1), (300, 136, 5), (4097, 1024, 64), (513, 7168, 8)])
 def test_bias_gather_add_matches_oracle(oracle, dev, dtype, ids_dtype, T, H, E):
     from atorch_amd.bias_gather_add import bias_gather_add_bw, bias_gather_add_fw
 
