@@ -113,8 +113,34 @@ struct Raw8<GLU> {
   }
 };
 
-// GELU on load (fp32 arithmetic of the torch op on a bf16 tensor, one rounding to bf16), and its
-// backward dh (cdf + x pdf) with cdf = (1 + erf(x / sqrt 2)) / 2, pdf = exp(-x^2 / 2) / sqrt(2 pi).
+// GELU on load, h = bf16(x Phi(x)), and its backward dh (Phi(x) + x pdf(x)), pdf = exp(-x^2 / 2) / sqrt(2 pi).
+// The reference evaluates Phi as (1 + erf(x / sqrt 2)) / 2 in fp32 (torch.nn.functional.gelu on a bf16 tensor).
+// Here Phi comes from the complementary function, without branches and without the cancellation of 1 + erf
+// for negative x:
+//   erfc(t) / 2 = exp(-t^2) q(u),  u = 1 / (1 + t / 2),  t = |x| / sqrt 2,
+// q a polynomial of degree 7 (a least-squares fit of erfcx(t) / 2 at Chebyshev nodes of u over 0 <= t <= 4.3,
+// relative error 6e-8; beyond 4.3, where erfc / 2 is below 1e-9, q stays at its value there), Phi(x) = erfc(t) / 2
+// for x < 0 and 1 - erfc(t) / 2 otherwise.  With s = |x| sqrt(log2(e) / 2) the exponential is exp2(-s^2) and
+// t / 2 = 0.41628 s: one v_rcp_f32, one v_exp_f32 and a dozen multiply-adds against the three divergent ranges of
+// the library's erff.  In fp32 arithmetic x Phi(x) comes out within 2.3e-6 of its value for |x| <= 6: rounded to
+// bf16 it equals the correctly rounded product for every normal bf16 x >= -4, and below that it keeps digits
+// where 1 + erf(x / sqrt 2) has lost them.  Infinities and NaNs give what the reference's formula gives.
+__device__ __forceinline__ float gelu_phi(float x, float* exp_neg_half_sq = nullptr) {
+  const float s = fabsf(x) * 0.8493217825889587f;  // sqrt(log2(e) / 2) |x|
+  const float u = __builtin_amdgcn_rcpf(__builtin_fmaf(fminf(s, 5.164826393127441f), 0.41627731919288635f, 1.0f));
+  float q = 0.042140234261751175f;
+  q = __builtin_fmaf(q, u, -0.16624070703983307f);
+  q = __builtin_fmaf(q, u, 0.1660318523645401f);
+  q = __builtin_fmaf(q, u, 0.05331931263208389f);
+  q = __builtin_fmaf(q, u, 0.11762023717164993f);
+  q = __builtin_fmaf(q, u, 0.14757198095321655f);
+  q = __builtin_fmaf(q, u, 0.13941511511802673f);
+  q = __builtin_fmaf(q, u, 0.00014206925698090345f);
+  const float e = __builtin_amdgcn_exp2f(-(s * s));  // exp(-x^2 / 2) = exp(-t^2)
+  if (exp_neg_half_sq) *exp_neg_half_sq = e;
+  const float h = q * e;  // erfc(t) / 2
+  return x < 0.f ? h : 1.0f - h;
+}
 template <>
 struct Raw8<GELU> {
   v4i a;
@@ -126,8 +152,8 @@ struct Raw8<GELU> {
     unpack8(a, x);
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
-      const float g0 = x[i] * 0.5f * (1.0f + erff(x[i] * 0.70710678118654752440f));
-      const float g1 = x[i + 1] * 0.5f * (1.0f + erff(x[i + 1] * 0.70710678118654752440f));
+      const float g0 = x[i] * gelu_phi(x[i]);
+      const float g1 = x[i + 1] * gelu_phi(x[i + 1]);
       const uint32_t h = pack_bf16x2(g0, g1);
       v[i] = __uint_as_float(h << 16);
       v[i + 1] = __uint_as_float(h & 0xffff0000u);
@@ -148,8 +174,9 @@ struct Raw8<GELUB> {
     unpack8(a, x);
     unpack8(d, g);
     auto grad = [](float xv, float gv) {
-      const float cdf = 0.5f * (1.0f + erff(xv * 0.70710678118654752440f));
-      const float pdf = 0.39894228040143267794f * __expf(-0.5f * xv * xv);
+      float e;  // exp(-x^2 / 2)
+      const float cdf = gelu_phi(xv, &e);
+      const float pdf = 0.39894228040143267794f * e;
       return gv * (cdf + xv * pdf);
     };
 #pragma unroll
@@ -310,9 +337,7 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
     if constexpr (kPacked) raw[i].pin();
     raw[i].get(vi);
     if constexpr (kPacked) {
-      v4i pk;
-      if constexpr (std::is_same<IN, BF16>::value) pk = raw[i].a;  // the input is the packed row
-      else pk = pack8_bf16(vi);
+      const v4i pk = pack8_bf16(vi);
 #pragma unroll
       for (int k = 0; k < 4; k++) vp[i][k] = (uint32_t)pk[k];
 #pragma unroll
