@@ -286,6 +286,13 @@ __device__ __forceinline__ void load_tile(const typename IN::elem* __restrict__ 
   for (int i = 0; i < 8; i++) raw[i].get(v[i]);
 }
 
+// Byte `b` of row `r` of the staged code tile.  A thread writes the few codes it holds of a row, and the lanes
+// c = 0..15 of a wave do so in rows eight apart: 8 * 144 bytes is a multiple of 128, so without more ado sixteen
+// lanes would meet in one or two LDS banks.  The 16-byte chunk index inside the row is therefore XORed with three
+// bits of the row: the 64 lanes of a write then spread evenly over all banks, and a row is still read back as
+// eight whole 16-byte chunks, in permuted order.
+__device__ __forceinline__ int staged_off(int r, int b) { return r * kTLd + (b ^ (((r >> 4) & 7) << 4)); }
+
 // the staged 128 x 128 code tile written as rows of 128 bytes, one 16-byte store per lane
 // (`out`: the tile's origin, the same in every lane; 128 ld_out < 2^32)
 __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t* __restrict__ out, uint32_t ld_out) {
@@ -294,7 +301,7 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
   for (int n = 0; n < 4; n++) {
     const int idx = (int)threadIdx.x + 256 * n;
     const int r = idx >> 3, ch = idx & 7;
-    st_nt(out, (uint32_t)r * ld_out + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(tile_t + r * kTLd + ch * 16));
+    st_nt(out, (uint32_t)r * ld_out + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(tile_t + staged_off(r, ch * 16)));
   }
 }
 
@@ -385,7 +392,7 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
       if constexpr (kPacked) col[i] = __uint_as_float(j & 1 ? vp[i][j / 2] & 0xffff0000u : vp[i][j / 2] << 16);
       else col[i] = v[i][j];
     }
-    *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = quant8(col, cdiv[j * 16 + c]);
+    *reinterpret_cast<v2i*>(tile_t + staged_off(c * 8 + j, gr * 8)) = quant8(col, cdiv[j * 16 + c]);
   }
   store_staged_tile(tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
 }
@@ -555,7 +562,7 @@ __device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa 
       float col[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) col[i] = __uint_as_float(j & 1 ? vp[w][i][j / 2] & 0xffff0000u : vp[w][i][j / 2] << 16);
-      *reinterpret_cast<int*>(&tile_t[w][(c * 8 + j) * kTLd + gr * 4]) = quant4(col, cdiv[w][j * 16 + c]);
+      *reinterpret_cast<int*>(&tile_t[w][staged_off(c * 8 + j, gr * 4)]) = quant4(col, cdiv[w][j * 16 + c]);
       if (j % 4 == 3) __builtin_amdgcn_sched_barrier(0);  // a few dividers at a time: sixteen of them are 64 registers
     }
   __syncthreads();
@@ -566,7 +573,7 @@ __device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa 
     for (int n = 0; n < 2; n++) {
       const int idx = tid + 512 * n;
       const int r = idx >> 3, ch = idx & 7;
-      st_nt(out, (uint32_t)r * ld_t + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(&tile_t[w][r * kTLd + ch * 16]));
+      st_nt(out, (uint32_t)r * ld_t + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(&tile_t[w][staged_off(r, ch * 16)]));
     }
   }
 }
@@ -671,7 +678,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
     v2i cols[8];
     transpose8x8_bytes(codes, cols);
 #pragma unroll
-    for (int j = 0; j < 8; j++) *reinterpret_cast<v2i*>(tile_t + (c * 8 + j) * kTLd + gr * 8) = cols[j];
+    for (int j = 0; j < 8; j++) *reinterpret_cast<v2i*>(tile_t + staged_off(c * 8 + j, gr * 8)) = cols[j];
     store_staged_tile(tile_t, q_t + (int64_t)e * N * K + (int64_t)kb * kTile * N + (int64_t)nb * kTile, (uint32_t)N);
   }
 }
