@@ -600,6 +600,10 @@ def run_quant(args, kernels, dev):
                                             M * F * (4 + 2 * q1), "2:1"),
         "swiglu_bwd_quant_1x128_dual_grouped": (lambda: kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E),
                                                 M * F * (6 + 4 * q1), "3:2"),
+        "gelu_quant_1x128_dual_grouped": (lambda: kernels.gelu_tile_quant_dual_grouped(x, goff, E),
+                                          M * F * (2 + 2 * q1), "1:1"),
+        "gelu_bwd_quant_1x128_dual_grouped": (lambda: kernels.gelu_tile_quant_dual_grouped(x, goff, E, dh=dh),
+                                              M * F * (4 + 2 * q1), "2:1"),
         "quant_128x128": (lambda: kernels.block_quant_batched(w), w.numel() * 3, "2:1"),
         "quant_128x128_with_transpose": (lambda: kernels.block_quant_batched(w, return_transpose=True),
                                          w.numel() * 4, "1:1"),
