@@ -874,6 +874,17 @@ def test_gelu_forward_and_backward_over_all_bf16_values(oracle, dev):
     _gelu_close(gr, oracle.gelu_bwd(dh, x), x)
     qo, so = oracle.tile_quant(gr.cpu())
     assert torch.equal(_u8(qb), qo) and torch.equal(sb.cpu(), so)
+    # Against the mathematics: x Phi(x) = x erfc(-x / sqrt 2) / 2 and Phi(x) + x pdf(x) evaluated in float64 and
+    # rounded once.  Where 1 + erf(x / sqrt 2) keeps its digits the kernels return exactly that value (the CPU op
+    # itself misses it on a few inputs).
+    xd = x.double()
+    phi = 0.5 * torch.special.erfc(-xd / 2.0**0.5)
+    want_h = (xd * phi).to(torch.bfloat16)
+    assert torch.equal(h.cpu()[x.float() >= -6.0], want_h[x.float() >= -6.0])
+    one = torch.ones_like(x)
+    gr1 = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, 1, dh=one.to(dev), return_activation=True)[4]
+    want_g = (phi + xd * torch.exp(-0.5 * xd * xd) / (2.0 * torch.pi) ** 0.5).to(torch.bfloat16)
+    assert torch.equal(gr1.cpu()[x.float() >= -4.0], want_g[x.float() >= -4.0])
 
 
 @pytest.mark.parametrize("backward", [False, True], ids=["fwd", "bwd"])
