@@ -1,5 +1,6 @@
-"""Seeded sweep of the grouped GEMMs over random shapes and routings against the float64 definition
-(triton_kernel.py:179-190 for one group; quantized_grouped_linear.py:243-253 for the weight gradient).
+"""Seeded sweeps over random shapes and routings: the grouped GEMMs against the float64 definition
+(triton_kernel.py:179-190 for one group; quantized_grouped_linear.py:243-253 for the weight gradient), and the
+row-wise + transposed quantisers of ragged groups against the oracle, bit for bit.
 
 The parametrised tests pick their shapes by hand; this one draws them: group counts from 1 to 130, empty
 groups, a few rows or tens of thousands (both tile configurations and every scale path of the kernel: batches
@@ -89,3 +90,59 @@ def test_grouped_gemms_on_random_shapes(seed):
         for e, m in enumerate(splits):
             if m == 0:  # an empty group: zeros, and with accumulation the old values untouched
                 assert dw[e].abs().max() == 0 and torch.equal(acc[e], base[e]), what
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_dual_quantisers_on_random_shapes(oracle, seed):
+    """Row-wise + transposed quantisation of ragged groups, plain and with the activations fused in, over drawn
+    shapes (triton_kernel.py:94-140 per row; the transposed codes follow quantized_grouped_linear.py:75-77 per
+    group).  Feature counts of 1024 and more take the workgroup order that deals eight neighbouring column
+    tiles to one XCD, with and without a remainder of token tiles outside that order."""
+    from atorch_amd import kernels
+
+    dev = torch.device("cuda:0")
+    rng = random.Random(seed)
+    for case in range(6):
+        F = TILE * rng.choice([1, 3, 8, 8, 16, 24])
+        E = rng.choice([1, 2, 3, 5, 9, 40])
+        M = rng.randint(1, 2500)
+        cuts = sorted(rng.randint(0, M) for _ in range(E - 1))
+        if E > 3 and rng.random() < 0.5:
+            cuts[1] = cuts[0]
+        bounds = [0] + cuts + [M]
+        splits = [bounds[i + 1] - bounds[i] for i in range(E)]
+        what = f"seed {seed} case {case}: M={M} F={F} E={E}"
+        print(what, flush=True)
+        g = torch.Generator().manual_seed(seed * 100 + case)
+        x = (torch.randn(M, F, generator=g) * torch.randn(M, 1, generator=g).exp()).bfloat16()
+        goff = kernels.group_offsets_from_splits(splits, dev)
+        ptot = oracle.padded_offsets(splits)[-1]
+
+        def same_as_plain(res, h):
+            # the fused kernel's codes and scales are those of the plain kernel on the fused kernel's own values
+            q, s, q_t, s_t = res
+            q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(h, goff, E, ld_t=q_t.shape[1])
+            assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2), what
+            assert torch.equal(q_t.view(torch.uint8)[:, :ptot], q_t2.view(torch.uint8)[:, :ptot]), what
+            assert torch.equal(s_t[: ptot // TILE], s_t2[: ptot // TILE]), what
+
+        q, s, q_t, s_t = kernels.tile_quant_dual_grouped(x.to(dev), goff, E)
+        qo, so = oracle.tile_quant(x)
+        qto, sto = oracle.tile_quant_t_grouped(x, splits, ld_t=q_t.shape[1])
+        assert torch.equal(q.view(torch.uint8).cpu(), qo) and torch.equal(s.cpu(), so), what
+        assert torch.equal(q_t.view(torch.uint8).cpu()[:, :ptot], qto[:, :ptot]), what
+        assert torch.equal(s_t.cpu()[: ptot // TILE], sto[: ptot // TILE]), what
+
+        fc1 = torch.cat([x, (torch.randn(M, F, generator=g)).bfloat16()], dim=1).contiguous().to(dev)
+        dh = (torch.randn(M, F, generator=g) * 0.1).bfloat16().to(dev)
+        *res, h = kernels.swiglu_tile_quant_dual_grouped(fc1, goff, E, return_activation=True)
+        same_as_plain(res, h)
+        *res, h = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, E, return_activation=True)
+        same_as_plain(res, h)
+        *res, gx = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, E, dh=dh, return_activation=True)
+        same_as_plain(res, gx)
+        *res, gfc1 = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E, return_grad=True)
+        same_as_plain(res, gfc1)
+        assert torch.equal(gfc1.cpu(), oracle.swiglu_bwd(dh.cpu(), fc1.cpu())) or rel_err(
+            gfc1.float().cpu(), oracle.swiglu_bwd(dh.cpu(), fc1.cpu()).float()
+        ) < 2.0**-6, what  # one or two bf16 units in the last place on a few inputs (hardware exp2 and reciprocal)
