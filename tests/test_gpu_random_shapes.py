@@ -1,6 +1,6 @@
 """Seeded sweeps over random shapes and routings: the grouped GEMMs against the float64 definition
 (triton_kernel.py:179-190 for one group; quantized_grouped_linear.py:243-253 for the weight gradient), and the
-row-wise + transposed quantisers of ragged groups against the oracle, bit for bit.
+row-wise + transposed quantisers of ragged groups and the dispatch kernels against the oracle, bit for bit.
 
 The parametrised tests pick their shapes by hand; this one draws them: group counts from 1 to 130, empty
 groups, a few rows or tens of thousands (both tile configurations and every scale path of the kernel: batches
@@ -146,3 +146,41 @@ def test_dual_quantisers_on_random_shapes(oracle, seed):
         assert torch.equal(gfc1.cpu(), oracle.swiglu_bwd(dh.cpu(), fc1.cpu())) or rel_err(
             gfc1.float().cpu(), oracle.swiglu_bwd(dh.cpu(), fc1.cpu()).float()
         ) < 2.0**-6, what  # one or two bf16 units in the last place on a few inputs (hardware exp2 and reciprocal)
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_dispatch_kernels_on_random_shapes(oracle, seed):
+    """Router preprocessing, the fused permute + quantise and the weighted combine over drawn token counts, widths,
+    expert counts and top-k (token_dispatcher.py:89-161), bit for bit against the oracle."""
+    from atorch_amd import kernels
+    from helpers import topk_routing
+
+    dev = torch.device("cuda:0")
+    rng = random.Random(seed)
+    for case in range(6):
+        E = rng.choice([2, 3, 8, 17, 64, 200])
+        k = rng.randint(1, min(E, 9))
+        T = rng.randint(1, 1500)
+        H = TILE * rng.choice([1, 2, 5, 8, 20, 40, 56])
+        probs_dtype = rng.choice([torch.bfloat16, torch.float32])
+        what = f"seed {seed} case {case}: T={T} H={H} E={E} k={k} probs={probs_dtype}"
+        print(what, flush=True)
+        g = torch.Generator().manual_seed(seed * 100 + case)
+        idx, probs = topk_routing(T, E, k, seed=seed * 100 + case, zipf_s=rng.choice([None, 1.2]))
+        probs = probs.to(probs_dtype)
+        x = (torch.randn(T, H, generator=g) * torch.randn(T, 1, generator=g).exp()).bfloat16()
+
+        sorted_idx, row_map, goff = kernels.moe_preprocess(idx.to(dev), E)
+        so, counts = oracle.permute_indices(idx, E)
+        assert torch.equal(sorted_idx.cpu(), so), what
+        assert torch.equal((goff[1:] - goff[:-1]).cpu(), counts.to(torch.int64)), what
+        q, s = kernels.permute_tile_quant(x.to(dev), row_map, k, T * k)
+        xp, _, _ = oracle.permute(x, idx, E)
+        qo, sco = oracle.tile_quant(xp)
+        assert torch.equal(q.view(torch.uint8).cpu(), qo) and torch.equal(s.cpu(), sco), what
+        assert torch.equal(kernels.permute_rows(x.to(dev), row_map, k, T * k).cpu(), xp), what
+
+        y = torch.randn(T * k, H, generator=g).bfloat16()
+        out = kernels.unpermute_combine(y.to(dev), row_map, probs.to(dev), T, k)
+        ref = oracle.unpermute(y, so, probs)
+        assert out.dtype == ref.dtype and torch.equal(out.cpu(), ref), what
