@@ -419,18 +419,18 @@ __global__ __launch_bounds__(256) void fill_zero_f32_kernel(float* __restrict__ 
   if (i < n) p[i] = 0.f;
 }
 
-// bgrad[e, :] += sum of the rows tagged e.  A workgroup walks kBgRows consecutive rows; a thread owns
-// one 16-byte chunk of columns and keeps the running sum of the current expert in registers, so rows
-// grouped by expert cost one set of atomics per workgroup and expert.
-constexpr int kBgRows = 128;
+// bgrad[e, :] += sum of the rows tagged e.  A workgroup walks rows_per_wg consecutive rows (a multiple of 8, chosen
+// by the launcher); a thread owns one 16-byte chunk of columns and keeps the running sum of the current expert in
+// registers, so rows grouped by expert cost one set of atomics per workgroup and expert.
+constexpr int kBgRowsMin = 32, kBgRowsMax = 4096;
 template <typename ID>
 __global__ __launch_bounds__(512) void bias_gather_bgrad_kernel(const v4i* __restrict__ grad, const ID* __restrict__ bin_ids,
                                                                 int64_t T, int row_chunks, int E, bool is_bf16,
-                                                                float* __restrict__ bgrad) {
+                                                                float* __restrict__ bgrad, int rows_per_wg) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= row_chunks) return;
-  const int64_t t0 = (int64_t)blockIdx.y * kBgRows;
-  const int64_t t1 = t0 + kBgRows < T ? t0 + kBgRows : T;
+  const int64_t t0 = (int64_t)blockIdx.y * rows_per_wg;
+  const int64_t t1 = t0 + rows_per_wg < T ? t0 + rows_per_wg : T;
   const int W = is_bf16 ? 8 : 4;  // columns per chunk
   float acc[8];
 #pragma unroll
@@ -530,16 +530,23 @@ extern "C" int aamd_bias_gather_add_bgrad(const void* grad, const void* bin_ids,
   if (T == 0) return AAMD_OK;
   AAMD_REQUIRE(grad && bin_ids, "bias_gather_add_bgrad: null pointer");
   AAMD_REQUIRE(((uintptr_t)grad & 15) == 0, "bias_gather_add_bgrad: grad must be 16-byte aligned");
-  const int64_t rc = row_bytes / 16, row_blocks = (T + kBgRows - 1) / kBgRows;
-  AAMD_REQUIRE(rc < 0x7fffffffLL && row_blocks <= 65535, "bias_gather_add_bgrad: more than 65535 * 128 rows");
+  const int64_t rc = row_bytes / 16;
   const int threads = threads_for_row_chunks(rc);
-  dim3 grid((unsigned)((rc + threads - 1) / threads), (unsigned)row_blocks), block((unsigned)threads);
+  // Rows per workgroup: every workgroup ends with one atomic add per column and expert it met, and those adds, not
+  // the reads, bound the launch when workgroups are short (128 rows each: 63 % of the HBM rate on 524288 x 7168
+  // bf16; 4096 rows each: 84 %).  About one workgroup per CU keeps enough loads in flight (half as many: 63 % again).
+  const int64_t col_blocks = (rc + threads - 1) / threads;
+  int64_t rows_per_wg = T * col_blocks / 256 / 8 * 8;
+  rows_per_wg = rows_per_wg < kBgRowsMin ? kBgRowsMin : rows_per_wg > kBgRowsMax ? kBgRowsMax : rows_per_wg;
+  const int64_t row_blocks = (T + rows_per_wg - 1) / rows_per_wg;
+  AAMD_REQUIRE(rc < 0x7fffffffLL && row_blocks <= 65535, "bias_gather_add_bgrad: more than 65535 * 4096 rows");
+  dim3 grid((unsigned)col_blocks, (unsigned)row_blocks), block((unsigned)threads);
   if (ids_are_i64)
     bias_gather_bgrad_kernel<int64_t><<<grid, block, 0, st>>>((const v4i*)grad, (const int64_t*)bin_ids, T, (int)rc, E,
-                                                              dtype == AAMD_BF16, bgrad);
+                                                              dtype == AAMD_BF16, bgrad, (int)rows_per_wg);
   else
     bias_gather_bgrad_kernel<int32_t><<<grid, block, 0, st>>>((const v4i*)grad, (const int32_t*)bin_ids, T, (int)rc, E,
-                                                              dtype == AAMD_BF16, bgrad);
+                                                              dtype == AAMD_BF16, bgrad, (int)rows_per_wg);
   AAMD_LAUNCH_CHECK("bias_gather_add_bgrad");
   return AAMD_OK;
 }
