@@ -46,28 +46,25 @@ __global__ __launch_bounds__(1024) void unpermute_combine_kernel(const typename 
     for (int a = 0; a < 4; a++)
 #pragma unroll
       for (int i = 0; i < VL; i++) acc[a][i] = 0.f;
-    // B gathered rows at a time: their loads are issued together, then folded in slot order.  (A
-    // plain loop over the slots compiles to one load in flight per lane.)  Streaming loads: a
+    // Eight gathered rows at a time: their loads are issued together, then folded in slot order.  (A plain loop
+    // over the slots compiles to one load in flight per lane.)  Row and weight are the same in every lane: held in
+    // scalar registers, the row address is scalar base + lane offset; slots past topk are skipped by branches the
+    // whole wave takes, a dropped copy contributes the zeros the reference multiplies there.  Streaming loads: a
     // permuted row is read exactly once.
-    auto batch = [&](auto Bc, int j0, auto A0c) {
-      constexpr int B = decltype(Bc)::value, A0 = decltype(A0c)::value;  // A0 = j0 mod 4
-      v4i raw[B];
-      float pv[B];
+    for (int j0 = 0; j0 < topk; j0 += 8) {
+      v4i raw[8];
+      float pv[8];
 #pragma unroll
-      for (int u = 0; u < B; u++) {
-        // row and weight are the same in every lane: held in scalar registers, the row address is
-        // scalar base + lane offset.  A dropped copy reads row 0 and is masked to the zeros the
-        // reference multiplies there.
-        const int r = __builtin_amdgcn_readfirstlane(srow[j0 + u]);
-        const int keep = r < 0 ? 0 : -1;
-        const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)(r < 0 ? 0 : r) * H) + c;  // H elements per row
-        raw[u] = __builtin_nontemporal_load(src);
-#pragma unroll
-        for (int i = 0; i < 4; i++) raw[u][i] &= keep;
-        pv[u] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(sprob[j0 + u])));
+      for (int u = 0; u < 8; u++) {
+        const bool on = j0 + u < topk;
+        const int r = on ? __builtin_amdgcn_readfirstlane(srow[on ? j0 + u : 0]) : -1;
+        pv[u] = on ? __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(sprob[on ? j0 + u : 0]))) : 0.f;
+        if (r >= 0) raw[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(y + (int64_t)r * H) + c);
+        else raw[u] = v4i{0, 0, 0, 0};
       }
 #pragma unroll
-      for (int u = 0; u < B; u++) {
+      for (int u = 0; u < 8; u++) {
+        if (j0 + u >= topk) break;
         float v[VL];
         if constexpr (kRowsF32) {
 #pragma unroll
@@ -88,21 +85,10 @@ __global__ __launch_bounds__(1024) void unpermute_combine_kernel(const typename 
             p0 = v[i] * pv[u];
             p1 = v[i + 1] * pv[u];
           }
-          acc[(A0 + u) & 3][i] = acc[(A0 + u) & 3][i] + p0;
-          acc[(A0 + u) & 3][i + 1] = acc[(A0 + u) & 3][i + 1] + p1;
+          acc[u & 3][i] = acc[u & 3][i] + p0;  // slot j0 + u, j0 a multiple of 8
+          acc[u & 3][i + 1] = acc[u & 3][i + 1] + p1;
         }
       }
-    };
-    using std::integral_constant;
-    int j = 0;  // stays a multiple of 4 until the batch of two
-    for (; j + 8 <= topk; j += 8) batch(integral_constant<int, 8>{}, j, integral_constant<int, 0>{});
-    if (j + 4 <= topk) { batch(integral_constant<int, 4>{}, j, integral_constant<int, 0>{}); j += 4; }
-    if (j + 2 <= topk) {
-      batch(integral_constant<int, 2>{}, j, integral_constant<int, 0>{});
-      j += 2;
-      if (j < topk) batch(integral_constant<int, 1>{}, j, integral_constant<int, 2>{});
-    } else if (j < topk) {
-      batch(integral_constant<int, 1>{}, j, integral_constant<int, 0>{});
     }
     float tot[VL];
 #pragma unroll
@@ -187,46 +173,87 @@ __global__ __launch_bounds__(256) void permute_rows_scaled_kernel(const typename
 
 // ---------------------------------------------------------------------------------------
 // gradient of the combine with respect to the weights: dprobs[t, j] = <dout[t], y[row_map[t*k+j]]>
-// (fp32 products and sums; one workgroup per token)
+// (fp32 products and sums).  One workgroup per token, as in the combine: a lane holds 8 columns of dout per trip
+// over the row, the gathers of up to eight slots are issued together, every lane keeps their partial sums, and the
+// workgroup reduces them once at the end (lanes of a wave by shuffles, waves in a fixed order through the LDS).
+// H8: columns / 8.
 // ---------------------------------------------------------------------------------------
 template <typename DT, typename YT>
-__global__ __launch_bounds__(256) void unpermute_probs_grad_kernel(const typename DT::elem* __restrict__ dout,
-                                                                   const typename YT::elem* __restrict__ y, int64_t M,
-                                                                   int64_t H, const int32_t* __restrict__ row_map,
-                                                                   int topk, float* __restrict__ dprobs) {
-  __shared__ float red[4];
+__global__ __launch_bounds__(1024) void unpermute_probs_grad_kernel(const typename DT::elem* __restrict__ dout,
+                                                                    const typename YT::elem* __restrict__ y, int64_t M,
+                                                                    int H8, const int32_t* __restrict__ row_map,
+                                                                    int topk, float* __restrict__ dprobs) {
+  constexpr bool kYF32 = std::is_same<YT, F32>::value;
+  __shared__ int srow[kMaxTopk];
+  __shared__ float red[16][kMaxTopk];
   const int64_t t = blockIdx.x;
-  auto load8 = [&](auto tag, const auto* p, float* v) {
-    using TT = decltype(tag);
-    if constexpr (std::is_same<TT, F32>::value) {
-      const v4f a = *reinterpret_cast<const v4f*>(p), b = *(reinterpret_cast<const v4f*>(p) + 1);
+  const int wave = (int)threadIdx.x >> 6, nwaves = (int)blockDim.x >> 6;
+  if ((int)threadIdx.x < topk) {
+    const int r = row_map[t * topk + threadIdx.x];
+    srow[threadIdx.x] = r >= 0 && r < M ? r : -1;  // a dropped copy: gradient 0
+  }
+  __syncthreads();
+  const int64_t H = (int64_t)H8 * 8;
+  for (int j0 = 0; j0 < topk; j0 += 8) {
+    float part[8];
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        v[i] = a[i];
-        v[4 + i] = b[i];
+    for (int u = 0; u < 8; u++) part[u] = 0.f;
+    for (int c = threadIdx.x; c < H8; c += blockDim.x) {
+      float a[8];
+      if constexpr (std::is_same<DT, F32>::value) {
+        const v4f lo = *reinterpret_cast<const v4f*>(dout + t * H + (int64_t)c * 8);
+        const v4f hi = *(reinterpret_cast<const v4f*>(dout + t * H + (int64_t)c * 8) + 1);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          a[i] = lo[i];
+          a[4 + i] = hi[i];
+        }
+      } else {
+        unpack8(*reinterpret_cast<const v4i*>(dout + t * H + (int64_t)c * 8), a);
       }
-    } else {
-      unpack8(*reinterpret_cast<const v4i*>(p), v);
-    }
-  };
-  for (int j = 0; j < topk; j++) {
-    const int64_t r = row_map[t * topk + j];
-    float part = 0.f;
-    if (r >= 0 && r < M) {
-      for (int64_t c = (int64_t)threadIdx.x * 8; c < H; c += 256 * 8) {
-        float a[8], b[8];
-        load8(DT{}, dout + t * H + c, a);
-        load8(YT{}, y + r * H + c, b);
+      v4i raw[8][kYF32 ? 2 : 1];
 #pragma unroll
-        for (int i = 0; i < 8; i++) part = part + a[i] * b[i];
+      for (int u = 0; u < 8; u++) {
+        // the row is the same in every lane (scalar base + lane offset); slots past topk and dropped copies are
+        // skipped by a branch the whole wave takes
+        const int r = j0 + u < topk ? __builtin_amdgcn_readfirstlane(srow[j0 + u < topk ? j0 + u : 0]) : -1;
+        const v4i* src = reinterpret_cast<const v4i*>(y + (int64_t)(r < 0 ? 0 : r) * H + (int64_t)c * 8);
+#pragma unroll
+        for (int w = 0; w < (kYF32 ? 2 : 1); w++) {
+          if (r >= 0) raw[u][w] = __builtin_nontemporal_load(src + w);
+          else raw[u][w] = v4i{0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if (j0 + u >= topk) break;
+        float b[8];
+        if constexpr (kYF32) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            b[i] = __int_as_float(raw[u][0][i]);
+            b[4 + i] = __int_as_float(raw[u][kYF32 ? 1 : 0][i]);
+          }
+        } else {
+          unpack8(raw[u][0], b);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) part[u] = part[u] + a[i] * b[i];
       }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
-    __syncthreads();
-    if (threadIdx.x == 0) dprobs[t * topk + j] = (red[0] + red[1]) + (red[2] + red[3]);
+    for (int u = 0; u < 8; u++) {
+      if (j0 + u >= topk) break;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) part[u] += __shfl_xor(part[u], off);
+      if ((threadIdx.x & 63) == 0) red[wave][j0 + u] = part[u];
+    }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < topk) {
+    float sum = 0.f;
+    for (int w = 0; w < nwaves; w++) sum += red[w][threadIdx.x];
+    dprobs[t * topk + threadIdx.x] = sum;
   }
 }
 
@@ -636,15 +663,26 @@ extern "C" int aamd_unpermute_probs_grad(const void* dout, int dout_dtype, const
   AAMD_REQUIRE(dout && row_map && dprobs && (y || M == 0), "unpermute_probs_grad: null pointer");
   AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)dout & 15) == 0, "unpermute_probs_grad: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)T), block(256);
+  if (M == 0) {  // every copy was dropped: no row to read (y may be null)
+    const int64_t n = T * topk;
+    AAMD_REQUIRE((n + 255) / 256 < 0x7fffffffLL, "unpermute_probs_grad: too large");
+    fill_zero_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(dprobs, n);
+    AAMD_LAUNCH_CHECK("unpermute_probs_grad (clear)");
+    return AAMD_OK;
+  }
+  // as few trips over the row as 1024 lanes allow, the lanes spread evenly over them (see aamd_unpermute_combine)
+  const int64_t chunks = H / 8, trips = (chunks + 1023) / 1024;
+  const int threads = H == 0 ? 64 : (int)(((chunks + trips - 1) / trips + 63) / 64 * 64);
+  const int H8 = (int)chunks;
+  dim3 grid((unsigned)T), block((unsigned)threads);
   if (dout_dtype == AAMD_BF16 && y_dtype == AAMD_BF16)
-    unpermute_probs_grad_kernel<BF16, BF16><<<grid, block, 0, st>>>((const u16*)dout, (const u16*)y, M, H, row_map, topk, dprobs);
+    unpermute_probs_grad_kernel<BF16, BF16><<<grid, block, 0, st>>>((const u16*)dout, (const u16*)y, M, H8, row_map, topk, dprobs);
   else if (dout_dtype == AAMD_F32 && y_dtype == AAMD_BF16)
-    unpermute_probs_grad_kernel<F32, BF16><<<grid, block, 0, st>>>((const float*)dout, (const u16*)y, M, H, row_map, topk, dprobs);
+    unpermute_probs_grad_kernel<F32, BF16><<<grid, block, 0, st>>>((const float*)dout, (const u16*)y, M, H8, row_map, topk, dprobs);
   else if (dout_dtype == AAMD_F32 && y_dtype == AAMD_F32)
-    unpermute_probs_grad_kernel<F32, F32><<<grid, block, 0, st>>>((const float*)dout, (const float*)y, M, H, row_map, topk, dprobs);
+    unpermute_probs_grad_kernel<F32, F32><<<grid, block, 0, st>>>((const float*)dout, (const float*)y, M, H8, row_map, topk, dprobs);
   else
-    unpermute_probs_grad_kernel<BF16, F32><<<grid, block, 0, st>>>((const u16*)dout, (const float*)y, M, H, row_map, topk, dprobs);
+    unpermute_probs_grad_kernel<BF16, F32><<<grid, block, 0, st>>>((const u16*)dout, (const float*)y, M, H8, row_map, topk, dprobs);
   AAMD_LAUNCH_CHECK("unpermute_probs_grad");
   return AAMD_OK;
 }
