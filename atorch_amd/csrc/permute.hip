@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const v4i* __restrict
                                                            const int32_t* __restrict__ row_map, int topk,
                                                            int64_t M_out, v4i* __restrict__ out) {
   const int64_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < chunks; c += 256) {
+  for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
     const v4i v = __builtin_nontemporal_load(x + t * chunks + c);
     for (int j = 0; j < topk; j++) {
       const int64_t dst = row_map[t * topk + j];
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void permute_rows_scaled_kernel(const typename
                                                                   const void* __restrict__ probs, int64_t M_out,
                                                                   typename OUT::elem* __restrict__ out) {
   const int64_t t = blockIdx.x;
-  for (int64_t c = (int64_t)threadIdx.x * 8; c < cols; c += 256 * 8) {
+  for (int64_t c = (int64_t)threadIdx.x * 8; c < cols; c += (int64_t)blockDim.x * 8) {
     float v[8];
     if constexpr (std::is_same<IN, F32>::value) {
       const v4f a = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + t * cols + c));
@@ -518,6 +518,16 @@ static int threads_for_row_chunks(int64_t chunks) {
   return threads;
 }
 
+// Workgroup size for the one-workgroup-per-token kernels, a lane handling one chunk of the row per trip: as few
+// trips as 1024 lanes allow, the lanes spread evenly over them, so that all the loads of a token are in flight at
+// once (7168 columns of bf16 in 16-byte chunks: 896 lanes and one trip; the combine runs at 74 % of the HBM rate
+// that way against 68 % with two trips of 448 lanes).
+static int threads_for_one_row(int64_t chunks) {
+  if (chunks <= 64) return 64;
+  const int64_t trips = (chunks + 1023) / 1024;
+  return (int)(((chunks + trips - 1) / trips + 63) / 64 * 64);
+}
+
 extern "C" int aamd_bias_gather_add(const void* inp, const void* bias, const void* bin_ids, int ids_are_i64, int64_t T,
                                     int64_t H, int E, int dtype, void* out, void* stream) {
   AAMD_REQUIRE(dtype == AAMD_BF16 || dtype == AAMD_F32, "bias_gather_add: unsupported dtype %d", dtype);
@@ -593,12 +603,8 @@ extern "C" int aamd_unpermute_combine(const void* y, int y_dtype, int64_t M, int
   AAMD_REQUIRE(probs_dtype == AAMD_NONE || probs != nullptr, "unpermute_combine: probs missing");
   AAMD_REQUIRE(((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0, "unpermute_combine: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  // one workgroup per token, one 16-byte chunk of the row per lane and trip.  As few trips as 1024 lanes allow, the
-  // lanes spread evenly over them: all gathers of a token are then in flight at once (7168 columns of bf16: 896 lanes
-  // and one trip, 74 % of the HBM rate against 68 % with two trips of 448).
-  const int64_t chunks = H / (y_dtype == AAMD_BF16 ? 8 : 4), trips = (chunks + 1023) / 1024;
-  const int threads = (int)(((chunks + trips - 1) / trips + 63) / 64 * 64);
-  dim3 grid((unsigned)T), block((unsigned)threads);
+  // one workgroup per token, one 16-byte chunk of the row per lane and trip
+  dim3 grid((unsigned)T), block((unsigned)threads_for_one_row(H / (y_dtype == AAMD_BF16 ? 8 : 4)));
   if (y_dtype == AAMD_BF16) {
     const int H8 = (int)(H / 8);
     if (probs_dtype == AAMD_BF16)
@@ -634,6 +640,7 @@ extern "C" int aamd_permute_rows_scaled(const void* x, int x_dtype, int64_t T, i
   AAMD_REQUIRE(x && out && row_map && (probs || probs_dtype == AAMD_NONE), "permute_rows_scaled: null pointer");
   AAMD_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "permute_rows_scaled: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
+  // (write bound: 256 lanes and several trips over the row measured faster at top-8 than one trip of up to 1024)
   dim3 grid((unsigned)T), block(256);
 #define AAMD_PRS(IN_, OUT_, PD_)                                                                                          \
   permute_rows_scaled_kernel<IN_, OUT_, PD_><<<grid, block, 0, st>>>((const IN_::elem*)x, cols, row_map, topk, probs, M_out, \
@@ -670,11 +677,8 @@ extern "C" int aamd_unpermute_probs_grad(const void* dout, int dout_dtype, const
     AAMD_LAUNCH_CHECK("unpermute_probs_grad (clear)");
     return AAMD_OK;
   }
-  // as few trips over the row as 1024 lanes allow, the lanes spread evenly over them (see aamd_unpermute_combine)
-  const int64_t chunks = H / 8, trips = (chunks + 1023) / 1024;
-  const int threads = H == 0 ? 64 : (int)(((chunks + trips - 1) / trips + 63) / 64 * 64);
-  const int H8 = (int)chunks;
-  dim3 grid((unsigned)T), block((unsigned)threads);
+  const int H8 = (int)(H / 8);
+  dim3 grid((unsigned)T), block((unsigned)threads_for_one_row(H8));
   if (dout_dtype == AAMD_BF16 && y_dtype == AAMD_BF16)
     unpermute_probs_grad_kernel<BF16, BF16><<<grid, block, 0, st>>>((const u16*)dout, (const u16*)y, M, H8, row_map, topk, dprobs);
   else if (dout_dtype == AAMD_F32 && y_dtype == AAMD_BF16)
