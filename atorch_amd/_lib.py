@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libatorch_amd_fp8.so")
 
 OK, ERR_ARG, ERR_HIP = 0, 1, 2
 NONE, BF16, F32, F16 = -1, 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib: Optional[ctypes.CDLL] = None
 
@@ -29,6 +29,10 @@ SIGNATURES = {
     "aamd_quant_1x128_dual_grouped": (
         _int,
         [_vp, _int, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _f32, _vp],
+    ),
+    "aamd_permute_quant_1x128_dual_grouped": (
+        _int,
+        [_vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _f32, _vp],
     ),
     "aamd_swiglu_quant_1x128": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     "aamd_swiglu_quant_1x128_dual_grouped": (
@@ -60,11 +64,6 @@ SIGNATURES = {
         _int,
         [_vp, _i64, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp],
     ),
-    "aamd_gemm_set_option": (_int, [ctypes.c_char_p, _int]),
-    "aamd_clock_probe": (_int, [_vp, _i64, _vp]),
-    "aamd_stream_probe": (_int, [_vp, _vp, _int, _int, _i64, _i64, _vp]),
-    "aamd_mfma_probe": (_int, [_vp, _int, _int, _int, _vp, _vp, _vp]),
-    "aamd_loop_probe": (_int, [_vp, _i64, _int, _int, _vp, _vp, _vp]),
     "aamd_unpermute_combine": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _i64, _int, _vp, _vp]),
     "aamd_permute_rows_scaled": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp, _int, _vp]),
     "aamd_unpermute_probs_grad": (_int, [_vp, _int, _vp, _int, _i64, _i64, _vp, _i64, _int, _vp, _vp]),

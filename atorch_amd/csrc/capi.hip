@@ -3,6 +3,9 @@
 #include <stdio.h>
 
 #include "common.hpp"
+#ifdef AAMD_TUNING
+#include "../../include/atorch_amd_probes.h"
+#endif
 
 namespace aamd {
 
@@ -22,5 +25,9 @@ int hip_fail(hipError_t e, const char* what) {
 
 }  // namespace aamd
 
+#ifndef AAMD_TUNING
 extern "C" int aamd_abi_version(void) { return AAMD_ABI_VERSION; }
 extern "C" const char* aamd_last_error(void) { return aamd::g_err; }
+#else  // the measurement library keeps its own error text
+extern "C" const char* aamd_probes_last_error(void) { return aamd::g_err; }
+#endif

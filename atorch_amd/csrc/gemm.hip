@@ -31,6 +31,9 @@
 #include <atomic>
 
 #include "common.hpp"
+#ifdef AAMD_TUNING
+#include "../../include/atorch_amd_probes.h"
+#endif
 
 namespace aamd {
 
@@ -117,6 +120,7 @@ struct Cfg {
 typedef Cfg<2, 2, 2, 2, 3> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two workgroups per CU
 typedef Cfg<2, 4, 4, 2, 1, true> CfgLarge;  // 512 threads, 256 (L) x 256 (R); one product buffer: 256 registers per lane
 typedef Cfg<2, 4, 2, 2> CfgWgrad;  // 512 threads, 256 (L) x 128 (R): room for the per-row R scales
+typedef Cfg<2, 4, 4, 2, 1> CfgWgrad256;  // 512 threads, 256 x 256, wave tiles of 128 (R) x 64 (L), one product buffer
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
 // expression inside the body.
@@ -506,7 +510,10 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     v8i lf[C::WTL][2];
     float cs[C::WTL];
     const float rblk = R_PER_ROW ? 1.f : Rsc[wrow0 / kTile];
-    v8i rf[2][2];
+    // R fragments: a ring of two sub-tile rows; with one product buffer and per-row scales (no registers to spare)
+    // one slot, refilled behind the last MFMAs that read it while that sub-tile's fold runs
+    constexpr int RF_SLOTS = R_PER_ROW && C::PRB == 1 ? 1 : 2;
+    v8i rf[RF_SLOTS][2];
     // LDS reads in the order of first use: the first MFMA waits for two fragments only, the rest
     // arrive in its shadow
     lf[0][0] = load_frag(la, BM, 0, 0);
@@ -524,22 +531,27 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       }
       cs[j] = Lsc[row * lsc_stride] * rblk;
     }
-    v4f rs[2][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
-    auto load_r = [&](int i) {
-      if (i > 0) {
-        rf[i & 1][0] = load_frag(ra, BN, i, 0);
-        rf[i & 1][1] = load_frag(ra, BN, i, 1);
-      }
+    // raw-product buffers: sub-tile t's fold runs D = PRB - 1 sub-tiles later (0: right after it).
+    // Per-row R scales live in a two-slot ring that allows at most D = 1; with D = 0 one slot is enough:
+    // the scales of an R row are read in front of its first MFMAs and used behind them.
+    constexpr int PRB = R_PER_ROW && C::PRB > 2 ? 2 : C::PRB;
+    constexpr int D = PRB - 1;
+    constexpr int RS_SLOTS = D == 0 ? 1 : 2;
+    v4f rs[RS_SLOTS][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
+    auto load_rs = [&](int i) {
       if constexpr (R_PER_ROW) {
 #pragma unroll
         for (int q = 0; q < 4; q++)
-          rs[i & 1][q] = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 32 + 8 * q + 4 * hg]);
+          rs[i % RS_SLOTS][q] = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 32 + 8 * q + 4 * hg]);
       }
     };
-    // raw-product buffers: sub-tile t's fold runs D = PRB - 1 sub-tiles later (0: right after it).
-    // Per-row R scales live in a two-slot ring that allows at most D = 1.
-    constexpr int PRB = R_PER_ROW && C::PRB > 2 ? 2 : C::PRB;
-    constexpr int D = PRB - 1;
+    auto load_r = [&](int i) {
+      if (i > 0) {
+        rf[i % RF_SLOTS][0] = load_frag(ra, BN, i, 0);
+        rf[i % RF_SLOTS][1] = load_frag(ra, BN, i, 1);
+      }
+      if constexpr (RS_SLOTS == 2) load_rs(i);
+    };
     v16f pr[PRB];
     load_r(0);
     // acc of sub-tile t += raw product * scales, registers [8*half, 8*half + 8) of the sub-tile
@@ -547,7 +559,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       const int i = t / C::WTL, j = t % C::WTL;
 #pragma unroll
       for (int r = 8 * half; r < 8 * half + 8; r++) {
-        const float sc = R_PER_ROW ? cs[j] * rs[i & 1][r / 4][r % 4] : cs[j];
+        const float sc = R_PER_ROW ? cs[j] * rs[i % RS_SLOTS][r / 4][r % 4] : cs[j];
         acc[i][j][r] = __builtin_fmaf(pr[t % PRB][r], sc, acc[i][j][r]);
       }
     };
@@ -561,12 +573,17 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       constexpr int t = decltype(T)::value;
       constexpr int i = t / C::WTL, j = t % C::WTL;
       __builtin_amdgcn_sched_barrier(0);
-      pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
+      if constexpr (RS_SLOTS == 1 && j == 0) load_rs(i);  // the last fold of the row before is done
+      pr[t % PRB] = mfma_fp8_32x32x64(rf[i % RF_SLOTS][0], lf[j][0], zero);
       __builtin_amdgcn_sched_barrier(0);
       if (D >= 1 && t >= D) fold_half(t - D, 0);
       __builtin_amdgcn_sched_barrier(0);
-      pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][1], lf[j][1], pr[t % PRB]);
+      pr[t % PRB] = mfma_fp8_32x32x64(rf[i % RF_SLOTS][1], lf[j][1], pr[t % PRB]);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (RF_SLOTS == 1 && j == C::WTL - 1 && i + 1 < C::WTR) {
+        load_r(i + 1);  // the row's last MFMAs have taken their operands; the fold below covers the reads
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (D >= 1 && t >= D) fold_half(t - D, 1);
       if (D == 0) {
         fold_half(t, 0);
@@ -574,7 +591,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       }
       __builtin_amdgcn_sched_barrier(0);
       // the next R row overwrites the fragment and scale slot of row i - 1, whose last fold is done
-      if (j == 0 && i + 1 < C::WTR) load_r(i + 1);
+      if (RF_SLOTS == 2 && j == 0 && i + 1 < C::WTR) load_r(i + 1);
       __builtin_amdgcn_sched_barrier(0);
       // every L fragment has been an MFMA operand by now, so it has left the LDS: the hook (a
       // barrier and the next L loads) costs no extra wait here
@@ -960,17 +977,17 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
 
 int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st);
 
-// Launch options a test or a tuning run may pin (aamd_gemm_set_option); -1 = the library chooses.
+// Launch choices a caller of the measurement build may pin per call (-1 = the library chooses, which is
+// all the product entry points ever pass).
 struct GemmOptions {
   int tile = -1;      // 0: 128x128 tiles, 1: the large configuration
   int group_r = -1;   // tile order groups R tiles (1) or L tiles (0)
   int gl = -1;        // tiles that share a panel in the tile order
   int ls_batch = -1;  // 0: L scales fetched one contraction block at a time
 };
-static GemmOptions g_opt;
 
 template <int MODE, bool R_PER_ROW, typename C>
-static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st) {
+static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st, const GemmOptions& g_opt) {
   if (blocks <= 0) return AAMD_OK;
   // L tiles per group of the tile order: 8 for the row-ragged launches; 4 for wgrad, whose operand
   // panels run over all tokens of an expert and are several times larger (measured: 5 % faster
@@ -981,7 +998,7 @@ static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st
   if (MODE == kRaggedK) p.group_r = p.nRt > p.nLt;
   else p.group_r = p.goff != nullptr && (int64_t)p.nRt * C::BM * p.E > p.Lrows;
   if (MODE == kRaggedRows && p.group_r) p.gl = 4;
-  // overrides set through aamd_gemm_set_option
+  // per-call overrides (measurement build only)
   if (g_opt.group_r >= 0) p.group_r = g_opt.group_r != 0 && (MODE == kRaggedK || p.goff != nullptr);
   if (g_opt.gl > 0) p.gl = g_opt.gl;
 
@@ -997,7 +1014,7 @@ static int launch_gemm(GemmParams p, int c_dtype, int64_t blocks, hipStream_t st
 
 // Tile choice: large tiles whenever the problem has enough of them to fill the chip
 // (option "tile": 0 forces the small configuration, 1 the large one).
-static bool use_large_tiles(int64_t tiles_256, bool by_default) {
+static bool use_large_tiles(int64_t tiles_256, bool by_default, const GemmOptions& g_opt) {
   if (g_opt.tile == 0) return false;
   if (g_opt.tile == 1) return true;
   // 256x256 tiles halve the bytes every CU pulls from L2 and measured faster wherever the launch
@@ -1011,19 +1028,10 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 using namespace aamd;
 
-extern "C" int aamd_gemm_set_option(const char* name, int value) {
-  AAMD_REQUIRE(name != nullptr, "gemm_set_option: null name");
-  if (!strcmp(name, "tile")) g_opt.tile = value;
-  else if (!strcmp(name, "group_r")) g_opt.group_r = value;
-  else if (!strcmp(name, "gl")) g_opt.gl = value;
-  else if (!strcmp(name, "ls_batch")) g_opt.ls_batch = value;
-  else AAMD_REQUIRE(false, "gemm_set_option: unknown option '%s'", name);
-  return AAMD_OK;
-}
-
 static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b, const float* b_s,
                         int b_tile_scaled, const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t M, int64_t N,
-                        int64_t K, void* c, int c_dtype, int64_t ldc, const void* bias, int bias_dtype, void* stream) {
+                        int64_t K, void* c, int c_dtype, int64_t ldc, const void* bias, int bias_dtype, void* stream,
+                        const GemmOptions& g_opt = GemmOptions()) {
   AAMD_REQUIRE(c_dtype == AAMD_BF16 || c_dtype == AAMD_F32, "grouped_gemm_nt: unsupported output dtype %d", c_dtype);
   AAMD_REQUIRE(M >= 0 && N >= 0 && K >= 0, "grouped_gemm_nt: negative size");
   AAMD_REQUIRE(K % kBK == 0 && N % kTile == 0, "grouped_gemm_nt: K=%lld and N=%lld must be multiples of 128",
@@ -1045,7 +1053,7 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   const bool batches16 = batches && (K / kBK) % 4 == 0 && aligned16(a_s);
   // tile-scaled B carries per-row R scales: use the configuration that has room for them; the 256x256
   // configuration takes all its scales in batches (with 4-byte loads where the rows are not aligned)
-  const bool large = use_large_tiles(((M + 255) / 256 + (group_offsets ? E : 0)) * ((N + 255) / 256), true) &&
+  const bool large = use_large_tiles(((M + 255) / 256 + (group_offsets ? E : 0)) * ((N + 255) / 256), true, g_opt) &&
                      (b_tile_scaled || batches);
   const int BM = large ? CfgLarge::BM : CfgSmall::BM;
   const int BN = large ? (b_tile_scaled ? CfgWgrad::BN : CfgLarge::BN) : CfgSmall::BN;
@@ -1069,12 +1077,13 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   const int64_t max_lt = group_offsets ? M / BM + E : (M + BM - 1) / BM;
   const int64_t blocks = max_lt * p.nRt;
   if (large)
-    return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgWgrad>(p, c_dtype, blocks, st)
-                         : launch_gemm<kRaggedRows, false, CfgLarge>(p, c_dtype, blocks, st);
-  return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgSmall>(p, c_dtype, blocks, st)
-                       : launch_gemm<kRaggedRows, false, CfgSmall>(p, c_dtype, blocks, st);
+    return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgWgrad>(p, c_dtype, blocks, st, g_opt)
+                         : launch_gemm<kRaggedRows, false, CfgLarge>(p, c_dtype, blocks, st, g_opt);
+  return b_tile_scaled ? launch_gemm<kRaggedRows, true, CfgSmall>(p, c_dtype, blocks, st, g_opt)
+                       : launch_gemm<kRaggedRows, false, CfgSmall>(p, c_dtype, blocks, st, g_opt);
 }
 
+#ifndef AAMD_TUNING
 extern "C" int aamd_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b,
                                         const float* b_s, int b_tile_scaled, const int64_t* group_offsets, int E,
                                         int32_t* tile_ws, int64_t M, int64_t N, int64_t K, void* c, int c_dtype,
@@ -1124,11 +1133,12 @@ extern "C" int aamd_grouped_gemm_fp8_nt_static(const uint8_t* a, int64_t lda, co
   return gemm_nt_impl(a, lda, a_s, b, b_s, b_tile_scaled, group_offsets, E, ws, M, N, K, c, c_dtype, ldc, bias,
                       bias_dtype, stream);
 }
+#endif  // !AAMD_TUNING
 
-extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt, const uint8_t* xt,
-                                           const float* sxt, int64_t ld_t, const int64_t* group_offsets, int E,
-                                           int32_t* tile_ws, int64_t N, int64_t K, void* dw, int dw_dtype,
-                                           int64_t expert_stride, int accumulate, void* stream) {
+static int wgrad_impl(const uint8_t* dyt, const float* sdyt, const uint8_t* xt, const float* sxt, int64_t ld_t,
+                      const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t N, int64_t K, void* dw,
+                      int dw_dtype, int64_t expert_stride, int accumulate, void* stream,
+                      const GemmOptions& g_opt = GemmOptions()) {
   AAMD_REQUIRE(dw_dtype == AAMD_BF16 || dw_dtype == AAMD_F32, "grouped_gemm_wgrad: unsupported output dtype %d", dw_dtype);
   AAMD_REQUIRE(N >= 0 && K >= 0 && N % kTile == 0 && K % kTile == 0,
                "grouped_gemm_wgrad: N=%lld and K=%lld must be multiples of 128", (long long)N, (long long)K);
@@ -1150,12 +1160,52 @@ extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt
   p.bias = nullptr; p.bias_dtype = AAMD_NONE; p.bias_group_stride = 0;
   p.goff = group_offsets; p.tile_off = tile_ws;
   // per-row scales on both operands: the 128x128 configuration measured faster for wgrad
-  const bool large = use_large_tiles(0, false);
-  const int BM = large ? CfgWgrad::BM : CfgSmall::BM, BN = large ? CfgWgrad::BN : CfgSmall::BN;
+  // (measurement build: tile 1 = 256 x 128, tile 2 = 256 x 256 with wave tiles of 128 x 64)
+  const int cfg = g_opt.tile > 0 ? g_opt.tile : 0;
+  const int BM = cfg ? CfgWgrad::BM : CfgSmall::BM;
+  const int BN = cfg == 2 ? CfgWgrad256::BN : cfg == 1 ? CfgWgrad::BN : CfgSmall::BN;
   p.Lrows = N; p.Rrows = K; p.nkb = 0; p.E = E; p.nRt = (int)((K + BN - 1) / BN); p.nLt = (int)((N + BM - 1) / BM);
   p.max_kb = (int)(ld_t / kBK);
   p.accumulate = accumulate;
   const int64_t blocks = (int64_t)E * p.nLt * p.nRt;
-  return large ? launch_gemm<kRaggedK, true, CfgWgrad>(p, dw_dtype, blocks, st)
-               : launch_gemm<kRaggedK, true, CfgSmall>(p, dw_dtype, blocks, st);
+#ifdef AAMD_TUNING
+  if (cfg == 2) return launch_gemm<kRaggedK, true, CfgWgrad256>(p, dw_dtype, blocks, st, g_opt);
+  if (cfg == 1) return launch_gemm<kRaggedK, true, CfgWgrad>(p, dw_dtype, blocks, st, g_opt);
+#endif
+  return launch_gemm<kRaggedK, true, CfgSmall>(p, dw_dtype, blocks, st, g_opt);
 }
+
+#ifndef AAMD_TUNING
+extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt, const uint8_t* xt,
+                                           const float* sxt, int64_t ld_t, const int64_t* group_offsets, int E,
+                                           int32_t* tile_ws, int64_t N, int64_t K, void* dw, int dw_dtype,
+                                           int64_t expert_stride, int accumulate, void* stream) {
+  return wgrad_impl(dyt, sdyt, xt, sxt, ld_t, group_offsets, E, tile_ws, N, K, dw, dw_dtype, expert_stride, accumulate,
+                    stream);
+}
+#else
+// Measurement build (libatorch_amd_probes.so): the same two GEMMs with the launch choices pinned per call.
+// opts = {tile, group_r, gl, ls_batch}, -1 = the library's own choice.
+extern "C" int aamd_tuning_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, const float* a_s, const uint8_t* b,
+                                               const float* b_s, int b_tile_scaled, const int64_t* group_offsets,
+                                               int E, int32_t* tile_ws, int64_t M, int64_t N, int64_t K, void* c,
+                                               int c_dtype, int64_t ldc, const void* bias, int bias_dtype,
+                                               const int* opts, void* stream) {
+  AAMD_REQUIRE(opts != nullptr, "tuning_grouped_gemm_nt: null options");
+  GemmOptions o;
+  o.tile = opts[0]; o.group_r = opts[1]; o.gl = opts[2]; o.ls_batch = opts[3];
+  return gemm_nt_impl(a, lda, a_s, b, b_s, b_tile_scaled, group_offsets, E, tile_ws, M, N, K, c, c_dtype, ldc, bias,
+                      bias_dtype, stream, o);
+}
+extern "C" int aamd_tuning_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt, const uint8_t* xt,
+                                                  const float* sxt, int64_t ld_t, const int64_t* group_offsets, int E,
+                                                  int32_t* tile_ws, int64_t N, int64_t K, void* dw, int dw_dtype,
+                                                  int64_t expert_stride, int accumulate, const int* opts,
+                                                  void* stream) {
+  AAMD_REQUIRE(opts != nullptr, "tuning_grouped_gemm_wgrad: null options");
+  GemmOptions o;
+  o.tile = opts[0]; o.group_r = opts[1]; o.gl = opts[2]; o.ls_batch = opts[3];
+  return wgrad_impl(dyt, sdyt, xt, sxt, ld_t, group_offsets, E, tile_ws, N, K, dw, dw_dtype, expert_stride, accumulate,
+                    stream, o);
+}
+#endif

@@ -1,6 +1,8 @@
-// Measurement aids of the library (no counterpart in the reference): the shader clock under load and
-// what the fp8 matrix pipes deliver from registers alone, with and without the block-scale fold.
+// Measurement aids (no counterpart in the reference), built into libatorch_amd_probes.so and never into the product
+// library: the shader clock under load, what the fp8 matrix pipes deliver from registers alone, with and without
+// the scale folds, a model of the GEMM's loop, and a streaming kernel for a given mix of read and written bytes.
 #include "common.hpp"
+#include "../../include/atorch_amd_probes.h"
 
 namespace aamd {
 
@@ -25,9 +27,10 @@ __global__ void clock_probe_kernel(unsigned long long* out, long long min_cycles
 
 // The GEMM's inner loop without any memory traffic: eight waves per workgroup (two per SIMD), each
 // with the fragments of a 128 x 64 wave tile in registers, issue per iteration the sixteen
-// v_mfma_f32_32x32x64_f8f6f4 of one 128-deep step.  FOLD: every pair's raw product is folded into the
-// accumulator with sixteen FMAs (the block-scale step); otherwise the MFMAs accumulate directly.
-template <bool FOLD>
+// v_mfma_f32_32x32x64_f8f6f4 of one 128-deep step.  FOLD 1: every pair's raw product is folded into the
+// accumulator with sixteen FMAs (the block-scale step); FOLD 2: with sixteen multiplies and sixteen FMAs
+// (per-row scales on both operands, the weight-gradient step); 0: the MFMAs accumulate directly.
+template <int FOLD>
 __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(const int* __restrict__ src, float* __restrict__ out,
                                                              int iters, unsigned long long* cyc) {
   const int tid = threadIdx.x;
@@ -49,17 +52,24 @@ __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(const int* __restric
 #pragma unroll
     for (int j = 0; j < 2; j++) acc[i][j] = zero;
   const float sc = 1.0f + 1e-7f * (float)(tid & 3);
+  v16f rs;  // per-row scales of the register axis (FOLD 2)
+#pragma unroll
+  for (int r = 0; r < 16; r++) rs[r] = 1.0f + 1e-7f * (float)((tid + r) & 7);
+  asm volatile("" : "+v"(rs));
   const unsigned long long t0 = __builtin_readcyclecounter();
   for (int it = 0; it < iters; it++) {
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
       for (int j = 0; j < 2; j++) {
-        if constexpr (FOLD) {
+        if constexpr (FOLD != 0) {
           v16f pr = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i][0], lf[j][0], zero, 0, 0, 0, 0, 0, 0);
           pr = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i][1], lf[j][1], pr, 0, 0, 0, 0, 0, 0);
 #pragma unroll
-          for (int r = 0; r < 16; r++) acc[i][j][r] = __builtin_fmaf(pr[r], sc, acc[i][j][r]);
+          for (int r = 0; r < 16; r++) {
+            if constexpr (FOLD == 2) acc[i][j][r] = __builtin_fmaf(pr[r], sc * rs[r], acc[i][j][r]);
+            else acc[i][j][r] = __builtin_fmaf(pr[r], sc, acc[i][j][r]);
+          }
         } else {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i][0], lf[j][0], acc[i][j], 0, 0, 0, 0, 0, 0);
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i][1], lf[j][1], acc[i][j], 0, 0, 0, 0, 0, 0);
@@ -310,10 +320,12 @@ extern "C" int aamd_mfma_probe(const void* operands, int fold, int iters, int wo
   AAMD_REQUIRE(iters >= 1 && iters <= (1 << 20) && workgroups >= 1 && workgroups <= (1 << 16), "mfma_probe: bad sizes");
   AAMD_REQUIRE((reinterpret_cast<uintptr_t>(operands) & 31) == 0, "mfma_probe: operands must be 32-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  if (fold)
-    aamd::mfma_probe_kernel<true><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
+  if (fold == 2)
+    aamd::mfma_probe_kernel<2><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
+  else if (fold)
+    aamd::mfma_probe_kernel<1><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
   else
-    aamd::mfma_probe_kernel<false><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
+    aamd::mfma_probe_kernel<0><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
   AAMD_LAUNCH_CHECK("mfma_probe");
   return AAMD_OK;
 }

@@ -308,11 +308,14 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
 // One 128 x 128 tile of the dual quantiser: token tile pt of group g, column tile kc.  Everything that
 // locates the tile is the same in every lane, so each access is a scalar base plus a 32-bit lane offset
 // (the launchers bound the row strides so that 128 rows stay below 2^32 bytes).
-template <typename IN, bool FULL>
+// GATHER: row r of the tile is source row src_row[r] of x (the token permute fused in: x is in token order,
+// the outputs in expert-contiguous order); src_row lives in LDS and holds every valid row of the tile.
+template <typename IN, bool FULL, bool GATHER = false>
 __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int nt, int64_t m0,
                                           int mvalid, int pt, int kc, uint8_t* __restrict__ q, float* __restrict__ s,
                                           uint8_t* __restrict__ q_t, float* __restrict__ s_t, uint32_t ld_t, float eps,
-                                          int64_t gate_off, u16* __restrict__ h_out, uint8_t* tile_t, Divider* cdiv) {
+                                          int64_t gate_off, u16* __restrict__ h_out, uint8_t* tile_t, Divider* cdiv,
+                                          const uint32_t* src_row = nullptr) {
   const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
   const int64_t cols = (int64_t)nt * kTile;
@@ -323,7 +326,19 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
   // inputs the 64 values of a thread stay in fp32: the packed form compiles to more registers there, not fewer.
   constexpr bool kPacked = std::is_same<IN, GELU>::value || std::is_same<IN, GELUB>::value;
   Raw8<IN> raw[8];
-  issue_tile_loads<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, raw, gate_off);
+  if constexpr (GATHER) {
+    // a row's 256-byte segment (16 lanes x 16 bytes) stays one coalesced access; only its base is looked up
+    constexpr uint32_t kEl = sizeof(typename IN::elem);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if (FULL || gr * 8 + i < mvalid)
+        raw[i].load(x + (int64_t)src_row[gr * 8 + i] * ldx + (int64_t)kc * kTile, (uint32_t)c * 8 * kEl, gate_off);
+      else
+        raw[i].zero();
+    }
+  } else {
+    issue_tile_loads<IN, FULL>(x + m0 * ldx + (int64_t)kc * kTile, ldx, mvalid, raw, gate_off);
+  }
   float v[kPacked ? 1 : 8][8];
   uint32_t vp[kPacked ? 8 : 1][4];
 
@@ -433,6 +448,50 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     dual_tile<IN, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, gate_off, h_out, tile_t, cdiv);
   else
     dual_tile<IN, false>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, gate_off, h_out, tile_t, cdiv);
+}
+
+// The dual quantiser with the token permute fused in: x holds the tokens in their original order, and permuted
+// row j (the rows of every output) is a copy of token sorted_idx[j] / topk, the stable order of the router
+// preprocess.  A workgroup looks up the source rows of its 128 permuted rows once (flat index / topk by a
+// multiply and a shift: magic = floor(2^sh / topk) + 1 with 2^(sh - 31) >= topk, exact for indices below 2^31)
+// and then runs the tile of the grouped kernel on gathered rows.  Source rows are clamped to the token count,
+// so a corrupt index reads a wrong row, never beyond x.
+template <typename IN>
+__global__ __launch_bounds__(256) void quant_dual_gather_kernel(
+    const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ sorted_idx,
+    uint32_t magic, int sh, uint32_t T, const int64_t* __restrict__ goff, const int32_t* __restrict__ tile_off, int E,
+    uint8_t* __restrict__ q, float* __restrict__ s, uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t,
+    float eps) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
+  __shared__ Divider cdiv[kTile];
+  __shared__ uint32_t src_row[kTile];
+  __shared__ int slot;
+  uint32_t bx = blockIdx.x, by = blockIdx.y;  // eight column tiles of a token tile on one XCD: see quant_dual_grouped_kernel
+  {
+    const uint32_t ntx = gridDim.x, per_row = ntx >> 3;
+    const uint32_t lin = by * ntx + bx, chunks = gridDim.y * per_row;
+    if ((ntx & 7) == 0 && lin < (chunks & ~7u) * 8) {
+      const uint32_t j = lin >> 3, chunk = (j & ~7u) + (lin & 7);
+      by = chunk / per_row;
+      bx = (chunk - by * per_row) * 8 + (j & 7);
+    }
+  }
+  const int pt = (int)by, kc = (int)bx;
+  const int g = __builtin_amdgcn_readfirstlane(find_group(tile_off, E, pt, &slot));
+  if (g >= E) return;
+  const int64_t m0 = goff[g] + (int64_t)(pt - tile_off[g]) * kTile;
+  const int64_t left = goff[g + 1] - m0;
+  const int mvalid = left < kTile ? (int)left : kTile;
+  if ((int)threadIdx.x < mvalid) {
+    const uint32_t flat = (uint32_t)sorted_idx[m0 + (int)threadIdx.x];
+    const uint32_t tok = (uint32_t)(((uint64_t)flat * magic) >> sh);
+    src_row[threadIdx.x] = tok < T ? tok : T - 1;
+  }
+  __syncthreads();
+  if (mvalid == kTile)
+    dual_tile<IN, true, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, 0, nullptr, tile_t, cdiv, src_row);
+  else
+    dual_tile<IN, false, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, 0, nullptr, tile_t, cdiv, src_row);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -683,35 +742,6 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const typename IN::e
   }
 }
 
-// tile_off[e] = sum_{j<e} ceil(rows_j / tile); one block, any E.
-__global__ __launch_bounds__(256) void group_tile_offsets_kernel(const int64_t* __restrict__ goff, int E, int tile,
-                                                                 int32_t* __restrict__ tile_off) {
-  __shared__ int buf[256];
-  __shared__ int carry;
-  if (threadIdx.x == 0) {
-    carry = 0;
-    tile_off[0] = 0;
-  }
-  __syncthreads();
-  for (int base = 0; base < E; base += 256) {
-    const int e = base + threadIdx.x;
-    int n = 0;
-    if (e < E) n = (int)((goff[e + 1] - goff[e] + tile - 1) / tile);
-    buf[threadIdx.x] = n;
-    __syncthreads();
-    for (int d = 1; d < 256; d <<= 1) {
-      int t = (int)threadIdx.x >= d ? buf[threadIdx.x - d] : 0;
-      __syncthreads();
-      buf[threadIdx.x] += t;
-      __syncthreads();
-    }
-    if (e < E) tile_off[e + 1] = carry + buf[threadIdx.x];
-    __syncthreads();
-    if (threadIdx.x == 255) carry += buf[255];
-    __syncthreads();
-  }
-}
-
 template <typename OUT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ q, const float* __restrict__ s,
                                                       int64_t M, int64_t N, int tile_scale,
@@ -751,11 +781,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
   }
 }
 
-int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st) {
-  group_tile_offsets_kernel<<<1, 256, 0, st>>>(goff, E, tile, tile_off);
-  AAMD_LAUNCH_CHECK("group_tile_offsets");
-  return AAMD_OK;
-}
+int launch_group_tile_offsets(const int64_t* goff, int E, int tile, int32_t* tile_off, hipStream_t st);
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -841,6 +867,49 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
   else
     quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
   AAMD_LAUNCH_CHECK("quant_dual_grouped");
+  return AAMD_OK;
+}
+
+extern "C" int aamd_permute_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
+                                                     const int64_t* sorted_idx, int topk, int64_t M,
+                                                     const int64_t* group_offsets, int E, int32_t* tile_ws, uint8_t* q,
+                                                     float* s, uint8_t* q_t, float* s_t, int64_t ld_t, float eps,
+                                                     void* stream) {
+  AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "permute_quant_dual: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(T >= 0 && M >= 0 && cols >= 0 && cols % kTile == 0, "permute_quant_dual: cols=%lld must be a multiple of 128",
+               (long long)cols);
+  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "permute_quant_dual: bad ldx=%lld", (long long)ldx);
+  AAMD_REQUIRE(topk >= 1 && topk <= 32768, "permute_quant_dual: topk=%d out of range", topk);
+  AAMD_REQUIRE(T * topk < ((int64_t)1 << 31) && M <= T * topk, "permute_quant_dual: T * topk must stay below 2^31 and M within it");
+  AAMD_REQUIRE(ld_t < kMaxTileLd && cols < kMaxTileLd, "permute_quant_dual: ld_t=%lld too large", (long long)ld_t);
+  AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "permute_quant_dual: group_offsets / tile_ws required");
+  AAMD_REQUIRE(ld_t % kTile == 0 && ld_t >= 0, "permute_quant_dual: ld_t=%lld must be a multiple of 128", (long long)ld_t);
+  AAMD_REQUIRE((q == nullptr) == (s == nullptr), "permute_quant_dual: q and s go together");
+  AAMD_REQUIRE(q_t && s_t, "permute_quant_dual: q_t / s_t required");
+  if (cols == 0 || M == 0) return AAMD_OK;
+  AAMD_REQUIRE(T > 0 && x && sorted_idx, "permute_quant_dual: null input");
+  const int64_t max_tiles = M / kTile + E;
+  const int64_t grid_tiles = ld_t / kTile < max_tiles ? ld_t / kTile : max_tiles;
+  if (grid_tiles == 0) return AAMD_OK;
+  AAMD_REQUIRE(aligned16(x) && aligned16(q_t) && (!q || aligned16(q)), "permute_quant_dual: pointers must be 16-byte aligned");
+  AAMD_REQUIRE(grid_tiles <= 65535, "permute_quant_dual: more than 65535 token tiles");
+  // flat / topk == (flat * magic) >> sh for flat < 2^31: magic = floor(2^sh / topk) + 1, sh = 31 + ceil(log2 topk)
+  int l = 0;
+  while ((1 << l) < topk) l++;
+  const int sh = 31 + l;
+  const uint32_t magic = (uint32_t)((((uint64_t)1 << sh) / (uint64_t)topk) + 1);
+  hipStream_t st = (hipStream_t)stream;
+  int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
+  if (rc) return rc;
+  dim3 grid((unsigned)(cols / kTile), (unsigned)grid_tiles), block(256);
+  const int nt = (int)(cols / kTile);
+  if (x_dtype == AAMD_BF16)
+    quant_dual_gather_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+  else if (x_dtype == AAMD_F16)
+    quant_dual_gather_kernel<F16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+  else
+    quant_dual_gather_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+  AAMD_LAUNCH_CHECK("permute_quant_dual_grouped");
   return AAMD_OK;
 }
 

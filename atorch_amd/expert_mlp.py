@@ -19,17 +19,33 @@ separately and their codes laid side by side, which makes the rest the merged ca
 Backward: the gradient through the activation is computed from the saved first-GEMM output by the
 kernel that quantises it (same fusion, autograd's bf16 arithmetic), and the four gradient GEMMs run
 on the fp8 kernels; bias gradients are per-expert fp32 row sums.
+
+Fused dispatch: with a ``TokenDispatch`` the hidden states come in token order and the permute of
+atorch/modules/moe/token_dispatcher.py:89-116 happens inside the quantiser of the first GEMM's operand
+(each permuted row is quantised straight from its token's row); the gradient of the hidden states goes
+back to token order through the sum over the top-k copies that ``index_select``'s backward makes there.
+The permuted bf16 rows are then neither written nor read, forward or backward.
 """
-from typing import Optional
+from typing import NamedTuple, Optional
 
 import torch
 
 from . import kernels
 from .bias_gather_add import bias_gather_add_bw
 from .gmm import _offsets
+from .quantization import WeightCodeCache
 
 
-def _quant_first_weight(w1, v1, transpose_w1):
+class TokenDispatch(NamedTuple):
+    """The routing of one batch as the device-side preprocess leaves it (``kernels.moe_preprocess``)."""
+
+    sorted_indices: torch.Tensor  # int64 [M]: flat (token * topk + slot) index of permuted row j
+    row_map: torch.Tensor  # int32 [T * topk]: permuted row of flat index i (-1: dropped copy)
+    topk: int
+    group_offsets: torch.Tensor  # int64 [E + 1]: exclusive prefix of permuted rows per expert
+
+
+def _quant_first_weight(w1, v1, transpose_w1, need_transpose=True):
     """Codes and scales of the first layer as the logical ``[E, N1, H]`` operand (N1 = 2F with SwiGLU) and
     its transpose ``[E, H, N1]``, from ``w1`` (and ``v1``) in either storage orientation."""
     q, s, q_t, s_t = kernels.block_quant_batched(w1.detach().contiguous(), return_transpose=True)
@@ -48,18 +64,32 @@ def _quant_first_weight(w1, v1, transpose_w1):
 
 class _Fp8ExpertMlp(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w1, w2, v1, b1, b2, batch_sizes, transpose_w1, activation):
+    def forward(ctx, x, w1, w2, v1, b1, b2, batch_sizes, transpose_w1, activation, dispatch, is_first_microbatch,
+                weight_cache):
         assert x.dim() == 2 and w1.dim() == 3 and w2.dim() == 3
         E = w1.shape[0]
-        goff = _offsets(batch_sizes, x.device)
-        train = any(t is not None and t.requires_grad for t in (x, w1, w2, v1, b1, b2))
+        goff = dispatch.group_offsets if dispatch is not None else _offsets(batch_sizes, x.device)
+        train = any(ctx.needs_input_grad)  # all False under no_grad
         glu = activation == "swiglu"
         # first weight(s) as [E, N1, H] (rows = outputs), second as [E, H, F]: block quantisation
         # commutes with the transpose, so both orientations come out of one launch each
-        q1, s1, q1_t, s1_t = _quant_first_weight(w1, v1, transpose_w1)
-        q2, s2, q2_t, s2_t = kernels.block_quant_batched(w2.detach().contiguous(), return_transpose=True)
+        quant1 = lambda t: _quant_first_weight(w1, v1, transpose_w1)  # noqa: E731
+        quant2 = lambda t: kernels.block_quant_batched(w2.detach().contiguous(), return_transpose=True)  # noqa: E731
+        if weight_cache is None:
+            (q1, s1, q1_t, s1_t), (q2, s2, q2_t, s2_t) = quant1(True), quant2(True)
+        else:
+            q1, s1, q1_t, s1_t = weight_cache.codes("w1", (w1, v1), is_first_microbatch, True, quant1)
+            q2, s2, q2_t, s2_t = weight_cache.codes("w2", (w2,), is_first_microbatch, True, quant2)
         xc = x.detach().contiguous()
-        if train:
+        if dispatch is not None:
+            M = dispatch.sorted_indices.numel()
+            if train:
+                qx, sx, qx_t, sx_t = kernels.permute_tile_quant_dual_grouped(
+                    xc, dispatch.sorted_indices, dispatch.topk, goff, E
+                )
+            else:  # every token quantised once, its codes written to its top-k rows
+                qx, sx = kernels.permute_tile_quant(xc, dispatch.row_map, dispatch.topk, M)
+        elif train:
             qx, sx, qx_t, sx_t = kernels.tile_quant_dual_grouped(xc, goff, E)
         else:
             qx, sx = kernels.tile_quant(xc)
@@ -76,12 +106,15 @@ class _Fp8ExpertMlp(torch.autograd.Function):
             ctx.transpose_w1, ctx.glu, ctx.has_v1 = transpose_w1, glu, v1 is not None
             ctx.has_b1, ctx.has_b2 = b1 is not None, b2 is not None
             ctx.dtypes = (x.dtype, w1.dtype, w2.dtype)
-            ctx.save_for_backward(goff, fc1, qx_t, sx_t, qh_t, sh_t, q1_t, s1_t, q2, s2)
+            ctx.dispatch_topk = dispatch.topk if dispatch is not None else 0
+            ctx.num_tokens = x.shape[0]
+            row_map = dispatch.row_map if dispatch is not None else goff
+            ctx.save_for_backward(goff, fc1, qx_t, sx_t, qh_t, sh_t, q1_t, s1_t, q2, s2, row_map)
         return out
 
     @staticmethod
     def backward(ctx, dy):
-        goff, fc1, qx_t, sx_t, qh_t, sh_t, q1_t, s1_t, q2, s2 = ctx.saved_tensors
+        goff, fc1, qx_t, sx_t, qh_t, sh_t, q1_t, s1_t, q2, s2, row_map = ctx.saved_tensors
         E = goff.numel() - 1
         x_dtype, w1_dtype, w2_dtype = ctx.dtypes
         dy = dy.contiguous().to(torch.bfloat16)
@@ -104,6 +137,8 @@ class _Fp8ExpertMlp(torch.autograd.Function):
         db1 = bias_gather_add_bw(res[4], bin_ids, E) if ctx.has_b1 else None
         # through the first linear: dx = dfc1 @ w1 ([M, H]); dw1[n, h] = sum_m dfc1[m, n] x[m, h]
         dx = kernels.grouped_gemm_nt(qg, sg, q1_t, s1_t, goff, out_dtype=x_dtype)
+        if ctx.dispatch_topk:  # back to token order: the sum over a token's copies (index_select's backward)
+            dx = kernels.unpermute_combine(dx, row_map, None, ctx.num_tokens, ctx.dispatch_topk)
         if ctx.transpose_w1:
             dw1 = kernels.grouped_gemm_wgrad(qg_t, sg_t, qx_t, sx_t, goff, out_dtype=w1_dtype)
         else:
@@ -112,27 +147,38 @@ class _Fp8ExpertMlp(torch.autograd.Function):
         if ctx.has_v1:  # the gate and the up half of the gradient go back to their own parameters
             dim = 1 if ctx.transpose_w1 else 2
             dw1, dv1 = (t.contiguous() for t in torch.chunk(dw1, 2, dim=dim))
-        return dx, dw1, dw2, dv1, db1, db2, None, None, None
+        return dx, dw1, dw2, dv1, db1, db2, None, None, None, None, None, None
 
 
-def grouped_mlp(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, tokens_per_expert: torch.Tensor,
-                v1: Optional[torch.Tensor] = None, b1: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None,
-                activation: str = "swiglu", transpose_w1: bool = True) -> torch.Tensor:
-    """The expert MLP on already permuted tokens: ``gmm -> (bias) -> activation -> gmm -> (bias)``.
+def grouped_mlp(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                tokens_per_expert: Optional[torch.Tensor], v1: Optional[torch.Tensor] = None,
+                b1: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None, activation: str = "swiglu",
+                transpose_w1: bool = True, *, dispatch: Optional[TokenDispatch] = None,
+                is_first_microbatch: Optional[bool] = None,
+                weight_cache: Optional[WeightCodeCache] = None) -> torch.Tensor:
+    """The expert MLP: ``gmm -> (bias) -> activation -> gmm -> (bias)``.
 
     ``hidden_states [M, H]`` bf16 rows grouped by expert; ``tokens_per_expert`` int64 ``[E]`` (CPU or
     device).  ``activation="swiglu"``: ``w1 [E, 2F, H]`` (merged gate / up), or ``w1`` and ``v1`` ``[E, F, H]``
     each; ``activation="gelu"``: ``w1 [E, F, H]``.  With ``transpose_w1=False`` the first weights are stored
     ``[E, H, *]``.  ``w2 [E, F, H]``; ``b1 [E, N1]`` / ``b2 [E, H]`` optional (not with ``v1``, as in the
-    reference).  H and F multiples of 128.  Returns ``[M, H]``."""
+    reference).  H and F multiples of 128.  Returns ``[M, H]``.
+
+    ``dispatch``: the permute fused in; ``hidden_states`` is then ``[T, H]`` in token order,
+    ``tokens_per_expert`` is not used (the dispatch carries the group offsets) and the result is the ``[M, H]``
+    expert output in permuted order, ready for the combine.  ``weight_cache`` / ``is_first_microbatch``: codes of
+    the weights kept between microbatches under the grouped linear's rule (``WeightCodeCache``); without a cache
+    the weights are quantised in every call."""
     assert hidden_states.dtype == torch.bfloat16, "the fused activation kernels read bf16"
     assert activation in ("swiglu", "gelu"), f"unknown activation {activation}"
     assert v1 is None or activation == "swiglu", "v1 is the up projection of a gated unit"
     assert v1 is None or (b1 is None and b2 is None), "bias not supported yet for not merge_w1_v1"
-    return _Fp8ExpertMlp.apply(hidden_states, w1, w2, v1, b1, b2, tokens_per_expert, transpose_w1, activation)
+    assert dispatch is not None or tokens_per_expert is not None, "tokens_per_expert or a dispatch is needed"
+    return _Fp8ExpertMlp.apply(hidden_states, w1, w2, v1, b1, b2, tokens_per_expert, transpose_w1, activation, dispatch,
+                               is_first_microbatch, weight_cache)
 
 
 def grouped_mlp_swiglu(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
-                       tokens_per_expert: torch.Tensor, transpose_w1: bool = True) -> torch.Tensor:
+                       tokens_per_expert: Optional[torch.Tensor], transpose_w1: bool = True, **kw) -> torch.Tensor:
     """``gmm -> SwiGLU -> gmm`` with the merged gate / up weight (``grouped_mlp`` with its defaults)."""
-    return grouped_mlp(hidden_states, w1, w2, tokens_per_expert, transpose_w1=transpose_w1)
+    return grouped_mlp(hidden_states, w1, w2, tokens_per_expert, transpose_w1=transpose_w1, **kw)

@@ -266,10 +266,19 @@ def _stack_of(ts) -> Optional[torch.Tensor]:
     equally spaced views of one buffer (the module's weights are); else None."""
     from .quantization import _base_of_stack
 
-    info = _base_of_stack(list(ts))
+    ts = list(ts)
+    info = _base_of_stack(ts)
     if info is None or info[1] != ts[0].numel():
         return None
-    return torch.as_strided(ts[0], (len(ts), *ts[0].shape), (ts[0].numel(), *ts[0].stride()))
+    # Adjacent addresses are not enough for a strided view: after module.to() / .bfloat16() /
+    # load_state_dict the tensors may sit side by side in memory and still own separate storages.
+    t0 = ts[0]
+    st0 = t0.untyped_storage()
+    if any(t.untyped_storage().data_ptr() != st0.data_ptr() for t in ts):
+        return None
+    if (t0.storage_offset() + len(ts) * t0.numel()) * t0.element_size() > st0.nbytes():
+        return None
+    return torch.as_strided(t0, (len(ts), *t0.shape), (t0.numel(), *t0.stride()))
 
 
 class _GroupedLinearDeviceOffsets(torch.autograd.Function):
@@ -295,6 +304,13 @@ class _GroupedLinearDeviceOffsets(torch.autograd.Function):
         kdt = torch.float32 if out_dtype == torch.float16 else out_dtype
 
         cached = getattr(module, "_stacked_weight_codes", None)
+        # one cache for both call forms: the stacked codes are valid only while the per-expert caches, which the
+        # m_splits form refreshes, still hold their slices
+        if cached is not None and any(
+            c.data is None or c.data.data_ptr() != cached[0][i].data_ptr()
+            for i, c in enumerate(module.weight_qresult_caches)
+        ):
+            cached = None
         update = is_first_microbatch or is_first_microbatch is None or force_quantize_per_microbatch()
         if update or cached is None or (is_grad_enabled and cached[2] is None):
             wstack = _stack_of([w.detach() for w in weights])

@@ -6,6 +6,7 @@ reference's functional surface (atorch/modules/fp8/triton_kernel.py:40,80,127,19
 grouped forms the grouped linear uses.  Every function enqueues HIP kernels on the current
 stream and returns torch tensors it allocated; nothing here computes on the CPU.
 """
+import threading
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -119,12 +120,15 @@ def fp8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Ten
     N = b.size(0)
     c = torch.empty(*a.size()[:-1], N, dtype=dtype, device=a.device)
     b_tile_scale = b_s.size(0) == b.size(0)
-    check(
-        lib().aamd_grouped_gemm_fp8_nt(
-            ptr(a), K, ptr(a_s), ptr(b), ptr(b_s), int(b_tile_scale), None, 1, None, M, N, K,
-            ptr(c), dtype_code(dtype), N, None, _lib.NONE, stream(),
-        )
-    )  # fmt: skip
+    args = (ptr(a), K, ptr(a_s), ptr(b), ptr(b_s), int(b_tile_scale), None, 1, None, M, N, K,
+            ptr(c), dtype_code(dtype), N, None, _lib.NONE)  # fmt: skip
+    pinned = _pinned_options()
+    if pinned:
+        from . import _probes
+
+        _probes.check(_probes.lib().aamd_tuning_grouped_gemm_fp8_nt(*args, _probes.options_array(pinned), stream()))
+    else:
+        check(lib().aamd_grouped_gemm_fp8_nt(*args, stream()))
     return c
 
 
@@ -193,6 +197,43 @@ def tile_quant_dual_grouped(
         lib().aamd_quant_1x128_dual_grouped(
             ptr(x), dtype_code(x.dtype, True), M, cols, cols, ptr(group_offsets), num_groups, ptr(ws),
             ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, eps, stream(),
+        )
+    )  # fmt: skip
+    return q, s, q_t, s_t
+
+
+def permute_tile_quant_dual_grouped(
+    x: torch.Tensor,
+    sorted_idx: torch.Tensor,
+    topk: int,
+    group_offsets: torch.Tensor,
+    num_groups: int,
+    eps: float = 0.0,
+    ld_t: Optional[int] = None,
+    rowwise: bool = True,
+):
+    """``tile_quant_dual_grouped`` of the permuted rows without materialising them: ``x [T, K]`` is in token
+    order, permuted row j is token ``sorted_idx[j] // topk`` (``sorted_idx`` int64 ``[M]`` from
+    ``moe_preprocess``).  Returns ``(q [M,K], s [M,K/128], q_t [K, ld_t], s_t [ld_t/128, K])``, bit-equal to
+    ``tile_quant_dual_grouped(permute_rows(x, ...), ...)``."""
+    assert x.dim() == 2 and x.is_contiguous()
+    T, cols = x.shape
+    assert cols % TILE == 0
+    assert sorted_idx.dtype == torch.int64 and sorted_idx.dim() == 1 and sorted_idx.is_contiguous()
+    M = sorted_idx.numel()
+    assert group_offsets.dtype == torch.int64 and group_offsets.numel() == num_groups + 1
+    if ld_t is None:
+        ld_t = padded_bound(M, num_groups)
+    dev = x.device
+    q = torch.empty((M, cols), dtype=FP8, device=dev) if rowwise else None
+    s = torch.empty((M, cols // TILE), dtype=torch.float32, device=dev) if rowwise else None
+    q_t = torch.empty((cols, ld_t), dtype=FP8, device=dev)
+    s_t = torch.empty((ld_t // TILE, cols), dtype=torch.float32, device=dev)
+    ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
+    check(
+        lib().aamd_permute_quant_1x128_dual_grouped(
+            ptr(x), dtype_code(x.dtype, True), T, cols, cols, ptr(sorted_idx), topk, M, ptr(group_offsets), num_groups,
+            ptr(ws), ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, eps, stream(),
         )
     )  # fmt: skip
     return q, s, q_t, s_t
@@ -382,13 +423,16 @@ def grouped_gemm_nt(
     ws = torch.empty(E + 1, dtype=torch.int32, device=a.device)
     if bias is not None:
         assert bias.shape == (E, N) and bias.is_contiguous()
-    check(
-        lib().aamd_grouped_gemm_fp8_nt(
-            ptr(a), a.stride(0), ptr(a_s), ptr(b), ptr(b_s), int(b_tile_scaled), ptr(group_offsets), E, ptr(ws),
+    args = (ptr(a), a.stride(0), ptr(a_s), ptr(b), ptr(b_s), int(b_tile_scaled), ptr(group_offsets), E, ptr(ws),
             M, N, K, ptr(out), dtype_code(out.dtype), out.stride(0),
-            ptr(bias), dtype_code(bias.dtype) if bias is not None else _lib.NONE, stream(),
-        )
-    )  # fmt: skip
+            ptr(bias), dtype_code(bias.dtype) if bias is not None else _lib.NONE)  # fmt: skip
+    pinned = _pinned_options()
+    if pinned:
+        from . import _probes
+
+        _probes.check(_probes.lib().aamd_tuning_grouped_gemm_fp8_nt(*args, _probes.options_array(pinned), stream()))
+    else:
+        check(lib().aamd_grouped_gemm_fp8_nt(*args, stream()))
     return out
 
 
@@ -416,12 +460,15 @@ def grouped_gemm_wgrad(
     assert out.shape == (E, N, K) and out.stride(2) == 1 and out.stride(1) == K
     ws = torch.empty(E + 1, dtype=torch.int32, device=dy_t.device)
     estride = out.stride(0) if E > 1 else N * K
-    check(
-        lib().aamd_grouped_gemm_fp8_wgrad(
-            ptr(dy_t), ptr(sdy_t), ptr(x_t), ptr(sx_t), ld_t, ptr(group_offsets), E, ptr(ws), N, K,
-            ptr(out), dtype_code(out.dtype), estride, int(accumulate), stream(),
-        )
-    )  # fmt: skip
+    args = (ptr(dy_t), ptr(sdy_t), ptr(x_t), ptr(sx_t), ld_t, ptr(group_offsets), E, ptr(ws), N, K,
+            ptr(out), dtype_code(out.dtype), estride, int(accumulate))  # fmt: skip
+    pinned = _pinned_options()
+    if pinned:
+        from . import _probes
+
+        _probes.check(_probes.lib().aamd_tuning_grouped_gemm_fp8_wgrad(*args, _probes.options_array(pinned), stream()))
+    else:
+        check(lib().aamd_grouped_gemm_fp8_wgrad(*args, stream()))
     return out
 
 
@@ -517,19 +564,33 @@ def split_views(t: torch.Tensor, splits: Sequence[int]) -> List[torch.Tensor]:
     return list(torch.split(t, list(splits)))
 
 
+_pinned = threading.local()  # launch options pinned by gemm_options on this thread
+
+
+def _pinned_options() -> Optional[dict]:
+    stack = getattr(_pinned, "stack", None)
+    return stack[-1] if stack else None
+
+
 class gemm_options:
-    """Context manager that pins launch choices of the grouped GEMMs (``aamd_gemm_set_option``) and
-    restores the library's own choice on exit: ``with gemm_options(tile=1): ...``."""
+    """Context manager for tests and tuning runs: inside it the grouped GEMMs of this thread go through the
+    measurement library's entry points (include/atorch_amd_probes.h), which take the launch choices as
+    per-call arguments: ``with gemm_options(tile=1): ...``.  Nested uses add to the enclosing one's options
+    and restore them on exit; nothing process-wide is changed and the product library is not involved."""
 
     def __init__(self, **opts):
+        from . import _probes
+
+        _probes.options_array(opts)  # validates the names
         self.opts = opts
 
     def __enter__(self):
-        for k, v in self.opts.items():
-            check(lib().aamd_gemm_set_option(k.encode(), int(v)))
+        if not hasattr(_pinned, "stack"):
+            _pinned.stack = []
+        outer = _pinned.stack[-1] if _pinned.stack else {}
+        _pinned.stack.append({**outer, **self.opts})
         return self
 
     def __exit__(self, *exc):
-        for k in self.opts:
-            check(lib().aamd_gemm_set_option(k.encode(), -1))
+        _pinned.stack.pop()
         return False

@@ -88,6 +88,41 @@ class QuantizeResultCache:
         return QuantizeResult(self.data, self.scale, self.data_t, self.scale_t)
 
 
+class WeightCodeCache:
+    """Block-quantised codes of expert weights kept between the microbatches of one optimizer step, for the
+    functional forms (``gmm``, ``grouped_mlp``) that have no module to hold ``QuantizeResultCache`` objects.
+
+    The rule is the module's (atorch/modules/fp8/quantized_grouped_linear.py:103-134): quantise when
+    ``is_first_microbatch`` is True or None, when the cached entry lacks the transposed codes a training call
+    needs, or when FORCE_QUANTIZE_PER_MICROBATCH is set (and then leave the cache alone); otherwise reuse.
+    Beyond the reference, an entry is also dropped when the weight it was made from has been written in place
+    or replaced since (its version counter, address, shape or dtype changed), so a forgotten
+    ``is_first_microbatch=True`` after an optimizer step cannot feed stale codes to the GEMMs."""
+
+    def __init__(self):
+        self._slots = {}
+
+    @staticmethod
+    def _stamp(tensors):
+        return tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype) for t in tensors if t is not None)
+
+    def codes(self, name: str, tensors, is_first_microbatch: Optional[bool], need_transpose: bool, quantise):
+        """``quantise(need_transpose) -> (q, s, q_t | None, s_t | None)`` for the weight tensors ``tensors``."""
+        force = force_quantize_per_microbatch()
+        slot = self._slots.get(name)
+        stamp = self._stamp(tensors)
+        update = is_first_microbatch or is_first_microbatch is None
+        if force or update or slot is None or slot[0] != stamp or (need_transpose and slot[1][2] is None):
+            codes = quantise(need_transpose)
+            if not force:
+                self._slots[name] = (stamp, codes)
+            return codes
+        return slot[1]
+
+    def clear(self):
+        self._slots.clear()
+
+
 @dataclass
 class QLinearParams:
     x_params: QParams = field(default_factory=lambda: QParams(quant_tile_shape=(1, TILE)))

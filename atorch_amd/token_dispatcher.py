@@ -146,14 +146,33 @@ class MoETokenDispatcher:
         return permuted, goff
 
     def token_permutation_fp8(self, hidden_states: torch.Tensor, max_prob: torch.Tensor, max_ind: torch.Tensor,
-                              eps: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-        """Forward only (codes have no gradient): ``(codes [M, H], scales [M, H/128], group_offsets)``."""
+                              eps: float = 0.0, return_transpose: bool = False):
+        """The permute fused into the 1x128 quantisation of the permuted rows, which are never written in bf16.
+        Codes have no gradient: this form feeds an inference forward, or a caller that handles the backward
+        itself (``expert_mlp.grouped_mlp(..., dispatch=self.dispatch())`` is the differentiable route).
+        Returns ``(codes [M, H], scales [M, H/128], group_offsets)``; with ``return_transpose`` (what a training
+        step's weight-gradient GEMM reads, quantized_grouped_linear.py:90-101 with ``is_grad_enabled``)
+        ``(codes, scales, codes_t [H, ld_t], scales_t [ld_t/128, H], group_offsets)`` in the layouts of
+        ``kernels.tile_quant_dual_grouped``."""
         self.hidden_shape = hidden_states.shape
         self.probs = max_prob
         x = _rows(hidden_states.detach())
-        goff = self.preprocess(max_ind)
+        self.preprocess(max_ind)  # a subclass may return tokens per expert: the prefix is self.group_offsets
+        if return_transpose:
+            q, s, q_t, s_t = kernels.permute_tile_quant_dual_grouped(
+                x, self.sorted_indices, self.topk, self.group_offsets, self.num_experts, eps=eps
+            )
+            return q, s, q_t, s_t, self.group_offsets
         q, s = kernels.permute_tile_quant(x, self.row_map, self.topk, self.row_map.numel(), eps=eps)
-        return q, s, goff
+        return q, s, self.group_offsets
+
+    def dispatch(self):
+        """The routing of the last ``preprocess`` as the ``TokenDispatch`` that ``expert_mlp.grouped_mlp`` takes to
+        fuse the permute into its first quantiser."""
+        from .expert_mlp import TokenDispatch
+
+        assert self.row_map is not None, "preprocess() first"
+        return TokenDispatch(self.sorted_indices, self.row_map, self.topk, self.group_offsets)
 
     def token_unpermutation(self, hidden_states: torch.Tensor, bias: torch.Tensor = None):
         assert bias is None, "Bias is not supported in MoETokenDispatcher"

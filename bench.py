@@ -20,8 +20,10 @@ stream; ``cpu_baseline`` is the reference's PyTorch CPU path (dequantise + per-e
 or the torch quantise / permute restatement) timed on this host on a bounded sample.
 """
 import argparse
+import hashlib
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -33,11 +35,32 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
 TILE = 128
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
-# this file (with --copy-probe: a plain 1 GiB copy reads FETCH_SIZE*2.0 KiB, WRITE_SIZE*1.0 KiB), averaged
-# over that kernel's launches of one step.  Counters cannot be read from inside the process, so the
-# figures are recorded here beside the profile summaries they come from (profiles/*.txt).
-MEASURED_TRAFFIC_BYTES = {"c2": 7.13e9, "c5": 4.830e9}
+# HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file
+# (with --copy-probe: a plain 1 GiB copy reads FETCH_SIZE*2.0 KiB, WRITE_SIZE*1.0 KiB), averaged over that kernel's
+# launches of one step.  Counters cannot be read from inside the process, so the figures are recorded in
+# profiles/hbm_traffic.json beside the profile summaries they come from, each with the SHA-256 of the kernel sources
+# it was measured on: a figure whose sources have changed since is not reported.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+CSRC = os.path.join(ROOT, "atorch_amd", "csrc")
+
+
+def source_hash(files):
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(CSRC, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def measured_traffic(key):
+    """Bytes per launch recorded for `key`, or None (with the reason) when there is no record for these sources."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))[key]
+    except (OSError, KeyError, ValueError):
+        return None, "no record in profiles/hbm_traffic.json"
+    if rec.get("source_sha256") != source_hash(rec["sources"]):
+        return None, f"stale: {', '.join(rec['sources'])} changed since {rec.get('profile')} was taken"
+    return rec["bytes_per_launch"], rec.get("profile")
 
 
 def parse():
@@ -78,7 +101,7 @@ def copy_probe(dev):
 # ------------------------------------------------------------------------------------------
 def clock_under(fn, dev, cycles=5_000_000):
     """Shader clock (GHz) read by a one-wave kernel on a second stream while fn()'s kernels run."""
-    from atorch_amd._lib import check, lib
+    from atorch_amd._probes import check, lib
 
     out = torch.zeros(2, dtype=torch.int64, device=dev)
     side = torch.cuda.Stream()
@@ -99,7 +122,7 @@ MIXES = ["1:0", "0:1", "1:1", "2:1", "1:2", "1:4", "4:1", "8:1", "3:2", "2:2"]
 
 def mix_probe(dev, mixes, stream_mib=512, iters=5):
     """GB/s of the streaming probe for each 'R:W' in mixes: R + W streams of stream_mib MiB each."""
-    from atorch_amd._lib import check, lib
+    from atorch_amd._probes import check, lib
 
     res = {}
     # streams one after the other, the stride kept off the powers of two: words of equal index in
@@ -131,7 +154,7 @@ def mix_probe(dev, mixes, stream_mib=512, iters=5):
 
 def mfma_probe(kernels, dev, iters=3000):
     """TFLOP/s of the GEMM's MFMA sequence issued from registers only, for three operand sets."""
-    from atorch_amd._lib import check, lib
+    from atorch_amd._probes import check, lib
 
     nbytes = 64 * 512 * 12 * 32
     g = torch.Generator(device=dev).manual_seed(7)
@@ -145,7 +168,7 @@ def mfma_probe(kernels, dev, iters=3000):
     cyc = torch.zeros(1, dtype=torch.int64, device=dev)
     res = {}
     for name, ops in sets.items():
-        for fold in (0, 1):
+        for fold in (0, 1, 2):  # 1: the block-scale fold (forward, dgrad); 2: per-row scales on both operands (wgrad)
             st = torch.cuda.current_stream().cuda_stream
             check(lib().aamd_mfma_probe(ops.data_ptr(), fold, iters, wgs, out.data_ptr(), cyc.data_ptr(), st))
             torch.cuda.synchronize()
@@ -156,7 +179,7 @@ def mfma_probe(kernels, dev, iters=3000):
             torch.cuda.synchronize()
             ms = a.elapsed_time(b)
             fl = wgs * 8 * iters * 16 * 131072.0
-            key = name + ("+fold" if fold else "")
+            key = name + ("", "+fold", "+fold_per_row")[fold]
             res[key] = {"TFLOP/s": round(fl / ms / 1e9, 1)}
             if fold:
                 # with the fold the two waves of a SIMD alternate on its pipe, so the probed wave runs for the
@@ -169,7 +192,7 @@ def loop_probe(dev, iters=2000):
     """One step of the 256 x 256 GEMM loop as an instruction sequence on private data (zero codes): shader
     cycles per step as one wave sees them (2048 of them are MFMA work) and TFLOP/s by the clock, with
     cache-resident loads, with loads that stream shared panels, and with the GEMM's barriers and waits."""
-    from atorch_amd._lib import check, lib
+    from atorch_amd._probes import check, lib
 
     panels = torch.zeros(16 * (96 << 20), dtype=torch.uint8, device=dev)  # 1.5 GiB: more than the last-level cache
     out = torch.empty(256 * 512, dtype=torch.float32, device=dev)
@@ -255,6 +278,13 @@ class Timer:
     def ms(self):
         return [a.elapsed_time(b) for a, b in self.pairs]
 
+    def mean(self):
+        ms = self.ms()
+        return sum(ms) / len(ms)
+
+    def median(self):
+        return statistics.median(self.ms())
+
 
 # ------------------------------------------------------------------------------------------
 # GEMM workloads
@@ -305,8 +335,11 @@ GEMM_WORKLOADS = {
 }  # fmt: skip
 
 
-def run_gemm(args, kernels, dev):
-    E, T, k, zipf, shapes, backward, desc = GEMM_WORKLOADS[args.workload]
+def run_gemm(args, kernels, dev, workload=None, steps=None, warmup=None, cpu_baseline=True, probes=True):
+    workload = workload or args.workload
+    steps = steps or args.steps
+    warmup = args.warmup if warmup is None else warmup
+    E, T, k, zipf, shapes, backward, desc = GEMM_WORKLOADS[workload]
     idx, _ = routing(T, E, k, dev, zipf_s=zipf)
     if zipf is not None:
         # the ragged configuration asks for empty groups: when the draw has none, the rarest expert's
@@ -350,26 +383,29 @@ def run_gemm(args, kernels, dev):
                 if timed:
                     b.record()
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step(False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step(True)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
 
     passes = 3 if backward else 1
     flops_step = passes * sum(L.flops for L in layers)
-    ms_step = dt * 1e3 / args.steps
+    ms_step = dt * 1e3 / steps
     tflops = flops_step / (ms_step * 1e-3) / 1e12
 
     # dominant kernel: the forward / dgrad grouped GEMM (4 of the 6 launches of a step)
-    nt_ms = nt_timer.ms()
     n_nt = len(layers) * (2 if backward else 1)
     nt_flops = sum(L.flops for L in layers) * (2 if backward else 1) / n_nt  # per launch, averaged
-    nt_avg_ms = sum(nt_ms) / len(nt_ms)
+    nt_avg_ms = nt_timer.mean()
     nt_tflops = nt_flops / (nt_avg_ms * 1e-3) / 1e12
+    # per-launch times of one step's launches differ by shape: the median is taken over steps of the per-step mean
+    per_step = [sum(nt_timer.ms()[i * n_nt : (i + 1) * n_nt]) / n_nt for i in range(steps)]
+    nt_med_ms = statistics.median(per_step)
+    traffic, traffic_src = measured_traffic("grouped_gemm_" + workload)
     roofline = {
         "kernel": "grouped_gemm_kernel<kRaggedRows> (forward and dgrad)",
         "bound": "mfma",
@@ -377,26 +413,31 @@ def run_gemm(args, kernels, dev):
         "peak": PEAK_FP8_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(nt_tflops / PEAK_FP8_TFLOPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+        "traffic": traffic,
+        "traffic_source": traffic_src,
         "avg_launch_ms": round(nt_avg_ms, 4),
+        "median_launch_ms": round(nt_med_ms, 4),
+        "achieved_by_median": round(nt_flops / (nt_med_ms * 1e-3) / 1e12, 2),
         "flop_per_launch": nt_flops,
     }
     extras = {"tokens_per_expert_min_max": [int(counts.min()), int(counts.max())],
               "empty_groups": int((counts == 0).sum()), "operands": args.operands}
-    extras["sclk_ghz_under_forward_gemm"] = clock_under(lambda: layers[0].fwd(kernels), dev)
+    if probes:
+        extras["sclk_ghz_under_forward_gemm"] = clock_under(lambda: layers[0].fwd(kernels), dev)
     if backward:
-        wg_ms = wg_timer.ms()
-        wg_avg = sum(wg_ms) / len(wg_ms)
+        wg_avg = wg_timer.mean()
         wg_flops = sum(L.flops for L in layers) / len(layers)
-        extras["wgrad_kernel"] = {"avg_launch_ms": round(wg_avg, 4),
+        n_wg = len(layers)
+        wg_med = statistics.median([sum(wg_timer.ms()[i * n_wg : (i + 1) * n_wg]) / n_wg for i in range(steps)])
+        extras["wgrad_kernel"] = {"avg_launch_ms": round(wg_avg, 4), "median_launch_ms": round(wg_med, 4),
                                   "achieved_tflops": round(wg_flops / (wg_avg * 1e-3) / 1e12, 2),
                                   "frac": round(wg_flops / (wg_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
 
-    if args.workload == "c2" and not args.no_extras and args.operands == "random":
+    if workload == "c2" and probes and not args.no_extras and args.operands == "random":
         extras["forward_gemm_by_operand_data"] = operand_data_probe(kernels, layers[0], dev)
 
     cpu = None
-    if not args.no_cpu_baseline and args.operands == "random":
+    if cpu_baseline and not args.no_cpu_baseline and args.operands == "random":
         cpu = cpu_gemm_baseline(layers[0], counts)
     return {
         "metric": "fp8 grouped-GEMM TFLOPS (fwd+bwd)" if backward else "fp8 grouped-GEMM TFLOPS (fwd)",
@@ -404,12 +445,56 @@ def run_gemm(args, kernels, dev):
         "unit": "TFLOP/s",
         "ms_per_step": round(ms_step, 4),
         "dtype": "fp8",
-        "config": {"workload": f"{args.workload}: {desc}", "rows": M, "experts": E,
+        "config": {"workload": f"{workload}: {desc}", "rows": M, "experts": E,
                    "flop_per_step": flops_step, "frac_of_fp8_peak": round(tflops / PEAK_FP8_TFLOPS, 4)},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "extras": extras,
     }  # fmt: skip
+
+
+def module_step(kernels, dev, steps=5):
+    """Forward + backward of the c2 expert MLP through the Python mirror (grouped_mlp_swiglu: quantisers, the fused
+    SwiGLU kernels and the six grouped GEMMs, host code included), the weights' codes cached as between the
+    microbatches of a step (quantized_grouped_linear.py:103-134)."""
+    from atorch_amd.expert_mlp import grouped_mlp_swiglu
+    from atorch_amd.quantization import WeightCodeCache
+
+    E, T, k, H, F = 8, 16384, 2, 4096, 14336
+    idx, _ = routing(T, E, k, dev)
+    _, _, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
+    counts = goff[1:] - goff[:-1]
+    M = T * k
+    x = randn((M, H), dev, 1.0, 1).requires_grad_(True)
+    w1 = randn((E, 2 * F, H), dev, 0.02, 2).requires_grad_(True)
+    w2 = randn((E, F, H), dev, 0.02, 3).requires_grad_(True)
+    dy = randn((M, H), dev, 1e-2, 4)
+    cache = WeightCodeCache()
+
+    def one(first):
+        out = grouped_mlp_swiglu(x, w1, w2, counts, is_first_microbatch=first, weight_cache=cache)
+        out.backward(dy)
+        x.grad = w1.grad = w2.grad = None
+
+    one(True)
+    one(False)
+    torch.cuda.synchronize()
+    res = {}
+    for name, first in (("cached_weight_codes", False), ("weights_quantised_every_call", None)):
+        t = Timer()
+        for _ in range(steps):
+            a, b = t.region()
+            a.record()
+            one(first)
+            b.record()
+        torch.cuda.synchronize()
+        fl = 3 * 2.0 * M * (2 * F * H + F * H)
+        res[name] = {"ms_per_step": round(t.mean(), 3), "median_ms": round(t.median(), 3),
+                     "TFLOP/s": round(fl / t.mean() / 1e9, 1), "frac_of_fp8_peak": round(fl / t.mean() / 1e9 / PEAK_FP8_TFLOPS, 4)}  # fmt: skip
+    res["what"] = "grouped_mlp_swiglu forward + backward at the c2 shapes: 2 + 3 quantiser launches and 6 grouped GEMMs"
+    del x, w1, w2, dy, cache
+    torch.cuda.empty_cache()
+    return res
 
 
 def operand_data_probe(kernels, layer, dev, iters=5):
@@ -474,14 +559,15 @@ def cpu_gemm_baseline(layer, counts):
 # ------------------------------------------------------------------------------------------
 # c5: quant / permute kernels
 # ------------------------------------------------------------------------------------------
-def run_c5(args, kernels, dev):
+def run_c5(args, kernels, dev, cpu_baseline=True, mixes_too=None):
     T, H, E, k = 65536, 7168, 64, 8
     x = student_t((T, H), dev, seed=0)
     idx, probs = routing(T, E, k, dev)
-    _, row_map, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
+    sorted_idx, row_map, goff = kernels.moe_preprocess(idx, E)
     M = T * k
     y = randn((M, H), dev, 1.0, seed=5)
     torch.cuda.synchronize()
+    q1 = 1 + 4 / TILE
     pq_bytes = T * H * 2 + M * H + M * (H // TILE) * 4 + M * 4
     uc_bytes = M * H * 2 + T * k * 2 + M * 4 + T * H * 2
     tq_bytes = M * H * 2 + M * H + M * (H // TILE) * 4
@@ -511,26 +597,57 @@ def run_c5(args, kernels, dev):
     dt = time.perf_counter() - t0
     ms_step = dt * 1e3 / args.steps
 
-    def gbs(nbytes, timer):
-        ms = timer.ms()
-        return nbytes / (sum(ms) / len(ms) * 1e-3) / 1e9, sum(ms) / len(ms)
+    def entry(nbytes, timer):
+        ms, med = timer.mean(), timer.median()
+        return {"GB/s": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                "avg_launch_ms": round(ms, 4), "median_launch_ms": round(med, 4), "bytes_per_launch": nbytes}  # fmt: skip
 
-    pq, pq_ms = gbs(pq_bytes, t_pq)
-    uc, uc_ms = gbs(uc_bytes, t_uc)
-    tq, tq_ms = gbs(tq_bytes, t_tq)
-    pre_ms = sum(t_pre.ms()) / len(t_pre.ms())
-    total_gbs = (pq_bytes + uc_bytes) / ((pq_ms + uc_ms) * 1e-3) / 1e9
+    pq, uc, tq = entry(pq_bytes, t_pq), entry(uc_bytes, t_uc), entry(tq_bytes, t_tq)
+    total_gbs = (pq_bytes + uc_bytes) / ((t_pq.mean() + t_uc.mean()) * 1e-3) / 1e9
+
+    # the training form: row-wise and transposed codes of the permuted rows.  Separate kernels write the permuted
+    # bf16 rows and read them back; the fused kernel quantises each permuted row straight from its token's row.
+    del y
+    torch.cuda.empty_cache()
+    t_sep, t_fused = Timer(), Timer()
+    for i in range(2 + 5):
+        for timer, fn in (
+            (t_sep, lambda: kernels.tile_quant_dual_grouped(kernels.permute_rows(x, row_map, k, M), goff, E)),
+            (t_fused, lambda: kernels.permute_tile_quant_dual_grouped(x, sorted_idx, k, goff, E)),
+        ):
+            a, b = timer.region() if i >= 2 else (None, None)
+            if a is not None:
+                a.record()
+            out = fn()
+            if b is not None:
+                b.record()
+            del out
+    torch.cuda.synchronize()
+    out_bytes = int(2 * M * H * q1)
+    dual = {
+        "permute_rows + quant_dual_grouped": {
+            "ms": round(t_sep.mean(), 4), "bytes_moved": T * H * 2 + 2 * M * H * 2 + out_bytes},
+        "permute_quant_dual_grouped (fused)": {
+            "ms": round(t_fused.mean(), 4), "bytes_moved": M * H * 2 + out_bytes,
+            "bytes_saved": T * H * 2 + M * H * 2,
+            "GB/s_of_bytes_moved": round((M * H * 2 + out_bytes) / t_fused.mean() / 1e6, 1),
+            "frac_of_bytes_moved": round((M * H * 2 + out_bytes) / t_fused.mean() / 1e6 / PEAK_HBM_GBS, 4)},
+        "note": "bytes_moved counts every token row once per top-k copy (the gather re-reads a token for each of its "
+                "experts' tiles; 0.94 GB of tokens do not stay in the 256 MB last-level cache between them)",
+    }  # fmt: skip
+
     cpu = None
-    if not args.no_cpu_baseline:
+    if cpu_baseline and not args.no_cpu_baseline:
         cpu = cpu_quant_baseline(x, idx)
     mixes = None
-    if args.workload == "c5" and not args.no_extras:
+    want_mixes = (args.workload == "c5" and not args.no_extras) if mixes_too is None else mixes_too
+    if want_mixes:
         # what plain streaming kernels reach with each kernel's ratio of bytes read to bytes written
-        del y
         torch.cuda.empty_cache()
         pr = mix_probe(dev, ["1:4", "8:1", "2:1"])
         mixes = {"permute_quant (1:4)": pr["1:4"]["GB/s"], "unpermute_combine (8:1)": pr["8:1"]["GB/s"],
                  "tile_quant_plain (2:1)": pr["2:1"]["GB/s"]}  # fmt: skip
+    traffic, traffic_src = measured_traffic("permute_quant_c5")
     return {
         "metric": "quant/permute HBM GB/s (permute+1x128 quant and unpermute+combine)",
         "value": round(total_gbs, 1),
@@ -541,16 +658,16 @@ def run_c5(args, kernels, dev):
                                "fused permute + 1x128 quant, and unpermute + weighted combine",
                    "rows": M, "experts": E},
         "roofline": {"kernel": "quant_1x128_kernel<bf16, scatter> (permute + quant)", "bound": "hbm",
-                     "achieved": round(pq, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(pq / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c5"),
-                     "avg_launch_ms": round(pq_ms, 4), "bytes_per_launch": pq_bytes},
+                     "achieved": pq["GB/s"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": pq["frac"], "traffic": traffic, "traffic_source": traffic_src,
+                     "avg_launch_ms": pq["avg_launch_ms"], "median_launch_ms": pq["median_launch_ms"],
+                     "bytes_per_launch": pq_bytes},
         "cpu_baseline": cpu,
         "extras": {
-            "unpermute_combine": {"GB/s": round(uc, 1), "frac": round(uc / PEAK_HBM_GBS, 4),
-                                  "avg_launch_ms": round(uc_ms, 4), "bytes_per_launch": uc_bytes},
-            "tile_quant_plain": {"GB/s": round(tq, 1), "frac": round(tq / PEAK_HBM_GBS, 4),
-                                 "avg_launch_ms": round(tq_ms, 4), "bytes_per_launch": tq_bytes},
-            "moe_preprocess_ms": round(pre_ms, 4),
+            "unpermute_combine": uc,
+            "tile_quant_plain": tq,
+            "permute_quant_dual (training form)": dual,
+            "moe_preprocess_ms": round(t_pre.mean(), 4),
             "mix_probe_GB/s": mixes,
         },
     }  # fmt: skip
@@ -581,7 +698,8 @@ def cpu_quant_baseline(x, idx):
 # ------------------------------------------------------------------------------------------
 # quant: the quantisation kernels of the expert MLP at the c2 shapes
 # ------------------------------------------------------------------------------------------
-def run_quant(args, kernels, dev):
+def run_quant(args, kernels, dev, steps=None, with_probe=True):
+    steps = steps or args.steps
     E, T, k, F = 8, 16384, 2, 14336
     idx, _ = routing(T, E, k, dev)
     _, _, goff = kernels.moe_preprocess(idx, E, want_sorted=False)
@@ -615,11 +733,11 @@ def run_quant(args, kernels, dev):
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        for _ in range(args.steps):
+        for _ in range(steps):
             fn()
         b.record()
         torch.cuda.synchronize()
-        ms = a.elapsed_time(b) / args.steps
+        ms = a.elapsed_time(b) / steps
         gbs = nbytes / ms / 1e6
         res[name] = {"GB/s": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4), "avg_launch_ms": round(ms, 4),
                      "bytes_per_launch": int(nbytes), "mix": mix}  # fmt: skip
@@ -627,10 +745,11 @@ def run_quant(args, kernels, dev):
         tot_ms += ms
     del x, fc1, dh, w
     torch.cuda.empty_cache()
-    probe = mix_probe(dev, sorted({v[2] for v in cases.values()}))
-    for name, (_, _, mix) in cases.items():
-        res[name]["mix_probe_GB/s"] = probe[mix]["GB/s"]
-        res[name]["frac_of_mix_probe"] = round(res[name]["GB/s"] / probe[mix]["GB/s"], 4)
+    if with_probe:
+        probe = mix_probe(dev, sorted({v[2] for v in cases.values()}))
+        for name, (_, _, mix) in cases.items():
+            res[name]["mix_probe_GB/s"] = probe[mix]["GB/s"]
+            res[name]["frac_of_mix_probe"] = round(res[name]["GB/s"] / probe[mix]["GB/s"], 4)
     worst = min(res, key=lambda n: res[n]["frac"])
     total = tot_b / tot_ms / 1e6
     return {
@@ -667,20 +786,45 @@ def main():
         res = run_quant(args, kernels, dev)
     else:
         res = run_c5(args, kernels, dev) if args.workload == "c5" else run_gemm(args, kernels, dev)
-    if args.workload == "c2" and not args.no_extras:
-        # the other half of the metric (quant / permute GB/s) and the two probes ride along in extras
+    if args.workload == "c2" and not args.no_extras and args.operands == "random":
+        # the other half of the metric (quant / permute GB/s), the other GEMM configurations, the module-level step and
+        # the probes ride along in extras; each is a short run of its own with the same timers
         torch.cuda.empty_cache()
-        args5 = argparse.Namespace(**{**vars(args), "no_cpu_baseline": True})
-        r5 = run_c5(args5, kernels, dev)
+        r5 = run_c5(args, kernels, dev, cpu_baseline=False, mixes_too=False)
         pq = r5["roofline"]
         res["extras"]["c5"] = {
-            "permute_quant": {"GB/s": pq["achieved"], "frac": pq["frac"], "avg_launch_ms": pq["avg_launch_ms"],
-                              "bytes_per_launch": pq["bytes_per_launch"]},
+            "permute_quant": {k: pq[k] for k in ("achieved", "frac", "avg_launch_ms", "median_launch_ms", "bytes_per_launch",
+                                                 "traffic")},
             "unpermute_combine": r5["extras"]["unpermute_combine"],
             "tile_quant_plain": r5["extras"]["tile_quant_plain"],
+            "permute_quant_dual (training form)": r5["extras"]["permute_quant_dual (training form)"],
         }  # fmt: skip
+        del r5
         torch.cuda.empty_cache()
+        rq = run_quant(args, kernels, dev, steps=10, with_probe=False)
+        res["extras"]["quant_kernels_c2_shapes"] = {
+            name: {k: v[k] for k in ("GB/s", "frac", "avg_launch_ms")} for name, v in rq["extras"]["kernels"].items()}
+        del rq
+        torch.cuda.empty_cache()
+        for wl in ("c3", "c4"):
+            r = run_gemm(args, kernels, dev, workload=wl, steps=10, warmup=3, cpu_baseline=False, probes=False)
+            res["extras"][wl] = {
+                "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                "frac_of_fp8_peak": r["config"]["frac_of_fp8_peak"],
+                "forward_dgrad_kernel_frac": r["roofline"]["frac"],
+                "empty_groups": r["extras"]["empty_groups"],
+                "tokens_per_expert_min_max": r["extras"]["tokens_per_expert_min_max"],
+                "wgrad_kernel": r["extras"].get("wgrad_kernel"),
+                "workload": r["config"]["workload"]}  # fmt: skip
+            del r
+            torch.cuda.empty_cache()
+        res["extras"]["module_step"] = module_step(kernels, dev)
         res["extras"]["mfma_probe"] = mfma_probe(kernels, dev)
+        # what the matrix pipes deliver on this operand data from registers alone, fold included: the ceiling the
+        # power limit leaves the kernel (the fraction above stays priced against the published 5.0 PFLOP/s)
+        lim = res["extras"]["mfma_probe"]["quantised_normal+fold"]["TFLOP/s"]
+        res["roofline"]["data_limited_ceiling_tflops"] = lim
+        res["roofline"]["frac_of_data_limited_ceiling"] = round(res["roofline"]["achieved"] / lim, 4)
         res["extras"]["loop_probe"] = loop_probe(dev)
     out = {
         "metric": res["metric"],

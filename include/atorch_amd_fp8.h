@@ -13,8 +13,8 @@
  *   - fp8 tensors are OCP e4m3fn codes, one byte each; scales are fp32
  *     dequantisation scales  s = max(amax, eps) / 448  (0 -> 1);
  *   - `dtype` arguments: AAMD_BF16 or AAMD_F32 (also AAMD_NONE where stated; the inputs of
- *     aamd_quant_1x128, aamd_permute_quant_1x128, aamd_quant_1x128_dual_grouped and
- *     aamd_quant_128x128 may also be AAMD_F16).
+ *     aamd_quant_1x128, aamd_permute_quant_1x128, aamd_quant_1x128_dual_grouped,
+ *     aamd_permute_quant_1x128_dual_grouped and aamd_quant_128x128 may also be AAMD_F16).
  *
  * Each entry point names the reference interface it replaces (paths relative
  * to the reference tree root).
@@ -27,6 +27,7 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+#pragma GCC visibility push(default) /* the entry points are the only symbols the library exports */
 
 #define AAMD_OK 0
 #define AAMD_ERR_ARG 1 /* bad shape / alignment / dtype */
@@ -37,7 +38,7 @@ extern "C" {
 #define AAMD_F32 1
 #define AAMD_F16 2 /* accepted as the input type of the quantisers only */
 
-#define AAMD_ABI_VERSION 2
+#define AAMD_ABI_VERSION 3
 
 /* Library identity and error text. */
 int aamd_abi_version(void);
@@ -93,6 +94,25 @@ int aamd_permute_rows(const void *x, int x_dtype, int64_t T, int64_t cols, const
 int aamd_quant_1x128_dual_grouped(const void *x, int x_dtype, int64_t M, int64_t cols, int64_t ldx,
                                   const int64_t *group_offsets, int E, int32_t *tile_ws, uint8_t *q, float *s,
                                   uint8_t *q_t, float *s_t, int64_t ld_t, float eps, void *stream);
+
+/*
+ * The token permute fused into aamd_quant_1x128_dual_grouped: x holds the tokens in their original order and
+ * every output row j (expert-contiguous order) is quantised from token sorted_idx[j] / topk, so the permuted
+ * bf16 rows are never written or re-read on the way to the grouped GEMMs of a training step.
+ * Replaces permute (atorch/modules/moe/token_dispatcher.py:89-116: argsort, index_select on sorted // topk)
+ * followed by the per-expert quantize_op.quantize(x_i, x_params, return_transpose=True) calls of
+ * atorch/modules/fp8/quantized_grouped_linear.py:90-101.
+ *   x [T, cols] (row stride ldx elements); sorted_idx [M] int64 (device): flat index token*topk+slot of
+ *   permuted row j, the sorted_idx of aamd_moe_preprocess (M < T*topk when copies were dropped);
+ *   T*topk < 2^31; group_offsets [E+1] int64 exclusive prefix of permuted rows per group;
+ *   q [M, cols], s [M, cols/128] (both may be NULL), q_t [cols, ld_t], s_t [ld_t/128, cols], tile_ws and ld_t
+ *   as for aamd_quant_1x128_dual_grouped.  Results equal aamd_permute_rows followed by
+ *   aamd_quant_1x128_dual_grouped bit for bit.
+ */
+int aamd_permute_quant_1x128_dual_grouped(const void *x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
+                                          const int64_t *sorted_idx, int topk, int64_t M,
+                                          const int64_t *group_offsets, int E, int32_t *tile_ws, uint8_t *q, float *s,
+                                          uint8_t *q_t, float *s_t, int64_t ld_t, float eps, void *stream);
 
 /*
  * 128x128 block quantisation of E weight matrices, optionally also emitting the
@@ -217,16 +237,6 @@ int aamd_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uin
                                 void *stream);
 
 /*
- * Pins a launch choice of the grouped GEMMs that the library otherwise makes by itself (for tests
- * and tuning runs; no counterpart in the reference).  value -1 restores the library's choice.
- *   "tile": 0 = 128x128 tiles, 1 = the large configuration; "group_r": tile order groups R tiles (1)
- *   or L tiles (0); "gl": tiles sharing a panel in the tile order; "ls_batch": 0 = scales fetched one
- *   contraction block at a time (which the 128x128 tiles do: the large configuration of the block-scaled GEMM takes
- *   its scales in batches only and is then not chosen).  Process-wide; not synchronised with running launches.
- */
-int aamd_gemm_set_option(const char *name, int value);
-
-/*
  * Inverse permutation + weighted combine in one gather-reduce pass:
  *   out[t, :] = sum_j probs[t, j] * y[row_map[t*topk + j], :]
  * Replaces unpermute, token_dispatcher.py:119-161 (zeros + index_copy_ + multiply + sum).
@@ -294,51 +304,7 @@ int aamd_bias_gather_add(const void *inp, const void *bias, const void *bin_ids,
 int aamd_bias_gather_add_bgrad(const void *grad, const void *bin_ids, int ids_are_i64, int64_t T, int64_t H, int E,
                                int dtype, float *bgrad, void *stream);
 
-/*
- * Shader clock probe (no counterpart in the reference; the benchmark reports the clock the GEMMs
- * run at): one wavefront spins for about min_cycles shader cycles (at most 2^31) and writes
- * out[0] = elapsed shader cycles, out[1] = elapsed ticks of the constant 100 MHz clock.
- */
-int aamd_clock_probe(uint64_t *out, int64_t min_cycles, void *stream);
-
-/*
- * Matrix-pipe probe (no counterpart in the reference; the benchmark reports what the fp8 MFMA pipes
- * deliver from registers alone, which on this GPU depends on the operand values through the power
- * limit): `workgroups` workgroups of eight waves issue, `iters` times, the sixteen
- * v_mfma_f32_32x32x64_f8f6f4 of one 128-deep step of a 128 x 64 wave tile, with the block-scale fold
- * (16 FMAs per MFMA pair) when fold != 0.  FLOP = workgroups * 8 * iters * 16 * 131072.
- *   operands: 64 * 512 * 12 * 32 bytes of fp8 codes (any values), 32-byte aligned
- *   out: workgroups * 512 floats (checksums); cycles[0]: shader cycles one wave spent in the loop.
- */
-int aamd_mfma_probe(const void *operands, int fold, int iters, int workgroups, float *out, uint64_t *cycles,
-                    void *stream);
-
-/*
- * Loop probe (no counterpart in the reference; the benchmark reports what one 128-deep step of the
- * 256 x 256 GEMM configuration costs as an instruction sequence on private data): 256 workgroups of
- * eight waves run, `iters` times, the step's sixteen MFMAs with their folds, its 24 fragment reads
- * from an LDS tile laid out like the GEMM's and its eight 1 KB direct-to-LDS loads, without scales,
- * barriers, prologue or epilogue.  stream_panels == 0: the loads re-read the first 4 KB of `panels`;
- * != 0: they walk 1 MiB panels (256 rows of 4 KB, 128 bytes per row and step) shared among the
- * workgroups of an XCD the way the GEMM's tiles share operand panels, and move on to the next set of
- * 96 panels every 32 steps (`panels` then holds a multiple of 96 MiB: panel_bytes / 96 MiB sets, wrapped);
- * 2: the same with the GEMM's two barriers per step, the wait for the loads of the step before in front
- * of the second one, and the loads issued where the GEMM issues them.
- * FLOP = 256 * 8 * iters * 16 * 131072; out: 256 * 512 floats; cycles[0]: shader cycles of one wave.
- */
-int aamd_loop_probe(const void *panels, int64_t panel_bytes, int stream_panels, int iters, float *out,
-                    uint64_t *cycles, void *stream);
-
-/*
- * Streaming probe (no counterpart in the reference; the benchmark prices the memory-bound kernels
- * against what the memory system delivers for their mix of read and written bytes): per 16-byte word
- * of work one word is read from each of `reads` input streams and one written to each of `writes`
- * output streams, all accesses streaming.  Stream i of src / dst starts at byte i * stride_bytes and
- * holds `units` words.  Built mixes: 1:0 0:1 1:1 2:1 1:2 1:4 4:1 8:1 3:2 2:2.
- */
-int aamd_stream_probe(const void *src, void *dst, int reads, int writes, int64_t stride_bytes, int64_t units,
-                      void *stream);
-
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

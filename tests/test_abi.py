@@ -9,10 +9,11 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "atorch_amd_fp8.h")
+PROBES_HEADER = os.path.join(ROOT, "include", "atorch_amd_probes.h")
 
 
-def _declared():
-    text = open(HEADER).read()
+def _declared(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(aamd_[a-z0-9_]+)\s*\(", text)))
 
@@ -37,11 +38,36 @@ def test_every_entry_point_cites_the_reference():
     text = open(HEADER).read()
     for block in re.findall(r"/\*(.*?)\*/\s*(?:int64_t|int)\s+(aamd_[a-z0-9_]+)\s*\(", text, flags=re.S):
         comment, name = block
-        if name in ("aamd_abi_version", "aamd_gemm_set_option"):
+        if name == "aamd_abi_version":
             continue
         if "no counterpart in the reference" in comment:
+            assert name == "aamd_grouped_gemm_fp8_nt_static", f"{name}: only the no-allocation entry may lack a counterpart"
             continue
         assert re.search(r"\.py:\d+", comment), f"{name}: no reference file:line in its comment"
+
+
+def test_product_library_exports_only_the_header_and_no_measurement_aid():
+    """Probes and launch-option pins live in libatorch_amd_probes.so; the product library exports exactly
+    the entry points of its header."""
+    import subprocess
+
+    from atorch_amd import _lib, _probes
+
+    out = subprocess.check_output(["nm", "-D", "--defined-only", _lib.LIB_PATH], text=True)
+    exported = sorted(ln.split()[-1] for ln in out.splitlines() if ln.split()[-1].startswith("aamd_"))
+    assert exported == _declared()
+    assert not any("probe" in n or "tuning" in n or "option" in n for n in exported)
+    P = _probes.lib()
+    names = _declared(PROBES_HEADER)
+    assert sorted(_probes.SIGNATURES) == names
+    for n in names:
+        assert hasattr(P, n), f"{n} declared in the probes header but not exported"
+    assert not set(names) & set(_declared()), "the two libraries share no entry point"
+    # the pinned GEMM validates like the product one, before touching the device
+    one = ctypes.c_void_p(16)
+    rc = P.aamd_tuning_grouped_gemm_fp8_nt(one, 64, one, one, one, 0, None, 1, None, 8, 128, 64, one, _lib.BF16, 128,
+                                           None, _lib.NONE, _probes.options_array({"tile": 1}), None)
+    assert rc == _lib.ERR_ARG and b"multiples of 128" in P.aamd_probes_last_error()
 
 
 def test_argument_validation_without_gpu():

@@ -381,6 +381,62 @@ def test_module_with_device_group_offsets_equals_host_splits(dev, bias, fuse):
         assert torch.equal(mods[1](x, None, group_offsets=goff, is_first_microbatch=False), oa.detach())
 
 
+def test_module_moved_to_the_device_runs_the_device_offset_path(dev):
+    """A module built on the CPU and moved with .to(): its weights (and main_grads taken one by one from the
+    allocator) may be adjacent in memory without sharing a storage.  The device-offset path and the fused
+    weight-gradient accumulation then take their fallbacks and give the bits of a module built on the device."""
+    from atorch_amd import kernels
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+
+    E, K, N = 3, 256, 128
+    splits = [100, 0, 156]
+    torch.manual_seed(6)
+    ref = ATorchGroupedLinear(E, K, N, bias=False, params_dtype=torch.bfloat16, device=dev, fuse_wgrad_accumulation=True)
+    mod = ATorchGroupedLinear(E, K, N, bias=False, params_dtype=torch.bfloat16, device="cpu", fuse_wgrad_accumulation=True)
+    with torch.no_grad():
+        for i in range(E):
+            mod.get_parameter(f"weight{i}").copy_(ref.get_parameter(f"weight{i}").cpu())
+    mod = mod.to(dev)
+    for m in (ref, mod):
+        for i in range(E):
+            m.get_parameter(f"weight{i}").main_grad = torch.full((N, K), 0.25, device=dev)
+    x = randn_bf16((sum(splits), K), 41).to(dev)
+    dy = randn_bf16((sum(splits), N), 42, std=1e-2).to(dev)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    outs = []
+    for m in (ref, mod):
+        xg = x.clone().requires_grad_(True)
+        for mb in (True, False):  # the second microbatch accumulates into main_grad
+            out = m(xg, None, group_offsets=goff, is_first_microbatch=mb)
+            out.backward(dy)
+        outs.append((out.detach(), xg.grad, [m.get_parameter(f"weight{i}").main_grad for i in range(E)]))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    for a, b in zip(outs[0][2], outs[1][2]):
+        assert torch.equal(a, b)
+    assert torch.all(outs[1][2][1] == 0)  # the empty group's gradient: written as zeros by the first microbatch
+
+
+def test_stacked_weight_codes_follow_the_per_expert_caches(dev):
+    """The two call forms of the module share one weight-code cache: after the m_splits form has requantised
+    (first microbatch of a new step), a group_offsets call with is_first_microbatch=False uses the new codes."""
+    from atorch_amd import kernels
+    from atorch_amd.grouped_linear import ATorchGroupedLinear
+
+    E, K, N = 2, 128, 128
+    splits = [64, 64]
+    torch.manual_seed(7)
+    mod = ATorchGroupedLinear(E, K, N, bias=False, params_dtype=torch.bfloat16, device=dev)
+    x = randn_bf16((128, K), 43).to(dev)
+    goff = kernels.group_offsets_from_splits(splits, dev)
+    with torch.no_grad():
+        mod(x, None, group_offsets=goff, is_first_microbatch=True)
+        for i in range(E):
+            mod.get_parameter(f"weight{i}").mul_(2.0)  # the optimizer step
+        want = mod(x, splits, is_first_microbatch=True)  # new step, host-split form: refreshes the per-expert caches
+        got = mod(x, None, group_offsets=goff, is_first_microbatch=False)
+    assert torch.equal(got, want)
+
+
 def test_module_accepts_fp16_activations(dev, oracle):
     """fp16 inputs and parameters (quantized_grouped_linear.py:533-534): codes and scales come from the fp16
     values exactly; outputs and gradients are fp16 and within the GEMM tolerance of the oracle."""

@@ -192,6 +192,42 @@ def test_weights_share_one_buffer_and_are_recognised():
     assert _base_of_rows(list(torch.split(wide, [30, 0, 50, 20]))) == (wide.data_ptr(), 128)
 
 
+def test_stack_view_needs_one_storage_not_only_adjacent_addresses():
+    """Tensors that sit side by side in memory but own separate storages (what module.to(), .bfloat16() or
+    load_state_dict into new parameters leave behind) cannot be viewed as one strided tensor: the helper
+    declines instead of raising, and callers fall back to a copy or a per-tensor loop."""
+    import numpy as np
+
+    from atorch_amd.grouped_linear import _stack_of
+    from atorch_amd.quantization import WeightCodeCache
+
+    mod = _module(3, 128, 128, bias=False)
+    ws = [getattr(mod, f"weight{i}").detach() for i in range(3)]
+    st = _stack_of(ws)
+    assert st is not None and st.shape == (3, 128, 128) and st.data_ptr() == ws[0].data_ptr()
+    raw = np.zeros(2 * 64 * 4, dtype=np.uint8)
+    a = torch.frombuffer(memoryview(raw)[: 64 * 4], dtype=torch.float32)
+    b = torch.frombuffer(memoryview(raw)[64 * 4 :], dtype=torch.float32)
+    assert b.data_ptr() == a.data_ptr() + 64 * 4  # adjacent, two storages
+    assert _stack_of([a, b]) is None
+    buf = torch.zeros(3 * 16)
+    assert _stack_of([buf[0:16], buf[16:32], buf[32:48]]) is not None
+    moved = _module(3, 128, 128, bias=False).to(torch.float64)  # every parameter gets a storage of its own
+    assert _stack_of([getattr(moved, f"weight{i}").detach() for i in range(3)]) is None
+    # the functional forms' cache: reuse only while the weight is unchanged
+    cache, calls = WeightCodeCache(), []
+    w = torch.zeros(4, 4)
+    make = lambda t: (calls.append(t), (1, 2, 3 if t else None, 4 if t else None))[1]  # noqa: E731
+    assert cache.codes("w", (w,), True, False, make) == (1, 2, None, None)
+    assert cache.codes("w", (w,), False, False, make) == (1, 2, None, None) and calls == [False]
+    assert cache.codes("w", (w,), False, True, make)[2] == 3 and calls == [False, True]  # transposes were missing
+    w.add_(1)
+    cache.codes("w", (w,), False, True, make)
+    assert calls == [False, True, True]  # written in place since: quantised again without being told
+    cache.codes("w", (w,), None, True, make)
+    assert len(calls) == 4  # None quantises on every call, like the module
+
+
 def test_transposed_layout_recognition():
     from atorch_amd.quantization import HipQuantizeOp
 

@@ -1,13 +1,15 @@
 """The entry point that allocates nothing, aamd_grouped_gemm_fp8_nt_static: the tile prefix lives in a
 static device array of the library instead of a caller workspace.  Called through the C ABI with raw
-ctypes and compared bit for bit with aamd_grouped_gemm_fp8_nt on the same operands, twice in a row,
-the second call on a smaller problem (fewer groups, fewer rows), so stale scratch contents would show."""
+ctypes and compared bit for bit with aamd_grouped_gemm_fp8_nt on the same operands and, within the GEMM
+tolerance, with the float64 dequantise-and-matmul definition, twice in a row: first a launch that takes the
+256 x 256 tiles (a prefix of 256-row tiles in the scratch), then a smaller one with fewer groups and rows on the
+128 x 128 tiles, so stale scratch contents would show."""
 import ctypes
 
 import pytest
 import torch
 
-from helpers import ragged_splits, randn_bf16
+from helpers import TILE, ragged_splits, randn_bf16, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -47,8 +49,9 @@ def test_static_scratch_entry_point_matches_the_workspace_one(dev):
     from atorch_amd import _lib
 
     L = _lib.lib()
-    # first a large-tile launch with many groups, then a smaller one with fewer groups and rows
-    for (M, N, K, E, seed, bias) in [(40000, 1024, 256, 130, 1, True), (700, 256, 384, 5, 2, False)]:
+    # first a large-tile launch with many groups (at least 512 tiles of 256 x 256 and eight contraction blocks
+    # select that configuration), then a smaller one with fewer groups and rows
+    for (M, N, K, E, seed, bias) in [(40000, 1024, 1024, 130, 1, True), (700, 256, 384, 5, 2, False)]:
         ops = _case(dev, M, N, K, E, seed, bias)
         assert 0 in ops[-1]
         ref = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=dev)
@@ -60,6 +63,17 @@ def test_static_scratch_entry_point_matches_the_workspace_one(dev):
         assert torch.cuda.mem_get_info()[0] == free_before, "the call must not allocate device memory"
         assert torch.equal(got, ref)
         assert not torch.all(got == 7.0)
+        # the definition, in float64 on the device: dequantised rows times the dequantised weight of their group
+        qx, sx, qw, sw, _, b, splits = ops
+        xd = (qx.float() * sx.repeat_interleave(TILE, 1)).double()
+        want = torch.full((M, N), 7.0, dtype=torch.float64, device=dev)
+        off = 0
+        for e, m in enumerate(splits):
+            if m:
+                wd = (qw[e].float() * sw[e].repeat_interleave(TILE, 0).repeat_interleave(TILE, 1)).double()
+                want[off : off + m] = xd[off : off + m] @ wd.t() + (b[e].double() if b is not None else 0.0)
+            off += m
+        assert rel_err(got.float().cpu(), want.float().cpu()) <= 1e-2
 
 
 def test_static_scratch_entry_point_rejects_too_many_groups(dev):
