@@ -120,7 +120,6 @@ struct Cfg {
 typedef Cfg<2, 2, 2, 2, 3> CfgSmall;  // 256 threads, 128 (L) x 128 (R), two workgroups per CU
 typedef Cfg<2, 4, 4, 2, 1, true> CfgLarge;  // 512 threads, 256 (L) x 256 (R); one product buffer: 256 registers per lane
 typedef Cfg<2, 4, 2, 2> CfgWgrad;  // 512 threads, 256 (L) x 128 (R): room for the per-row R scales
-typedef Cfg<2, 4, 4, 2, 1> CfgWgrad256;  // 512 threads, 256 x 256, wave tiles of 128 (R) x 64 (L), one product buffer
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant
 // expression inside the body.
@@ -510,10 +509,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     v8i lf[C::WTL][2];
     float cs[C::WTL];
     const float rblk = R_PER_ROW ? 1.f : Rsc[wrow0 / kTile];
-    // R fragments: a ring of two sub-tile rows; with one product buffer and per-row scales (no registers to spare)
-    // one slot, refilled behind the last MFMAs that read it while that sub-tile's fold runs
-    constexpr int RF_SLOTS = R_PER_ROW && C::PRB == 1 ? 1 : 2;
-    v8i rf[RF_SLOTS][2];
+    v8i rf[2][2];
     // LDS reads in the order of first use: the first MFMA waits for two fragments only, the rest
     // arrive in its shadow
     lf[0][0] = load_frag(la, BM, 0, 0);
@@ -531,27 +527,22 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       }
       cs[j] = Lsc[row * lsc_stride] * rblk;
     }
-    // raw-product buffers: sub-tile t's fold runs D = PRB - 1 sub-tiles later (0: right after it).
-    // Per-row R scales live in a two-slot ring that allows at most D = 1; with D = 0 one slot is enough:
-    // the scales of an R row are read in front of its first MFMAs and used behind them.
-    constexpr int PRB = R_PER_ROW && C::PRB > 2 ? 2 : C::PRB;
-    constexpr int D = PRB - 1;
-    constexpr int RS_SLOTS = D == 0 ? 1 : 2;
-    v4f rs[RS_SLOTS][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
-    auto load_rs = [&](int i) {
+    v4f rs[2][4];  // R_PER_ROW: scales of the 16 R rows this lane holds in a sub-tile
+    auto load_r = [&](int i) {
+      if (i > 0) {
+        rf[i & 1][0] = load_frag(ra, BN, i, 0);
+        rf[i & 1][1] = load_frag(ra, BN, i, 1);
+      }
       if constexpr (R_PER_ROW) {
 #pragma unroll
         for (int q = 0; q < 4; q++)
-          rs[i % RS_SLOTS][q] = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 32 + 8 * q + 4 * hg]);
+          rs[i & 1][q] = *reinterpret_cast<const v4f*>(&Rsc[wrow0 + i * 32 + 8 * q + 4 * hg]);
       }
     };
-    auto load_r = [&](int i) {
-      if (i > 0) {
-        rf[i % RF_SLOTS][0] = load_frag(ra, BN, i, 0);
-        rf[i % RF_SLOTS][1] = load_frag(ra, BN, i, 1);
-      }
-      if constexpr (RS_SLOTS == 2) load_rs(i);
-    };
+    // raw-product buffers: sub-tile t's fold runs D = PRB - 1 sub-tiles later (0: right after it).
+    // Per-row R scales live in a two-slot ring that allows at most D = 1.
+    constexpr int PRB = R_PER_ROW && C::PRB > 2 ? 2 : C::PRB;
+    constexpr int D = PRB - 1;
     v16f pr[PRB];
     load_r(0);
     // acc of sub-tile t += raw product * scales, registers [8*half, 8*half + 8) of the sub-tile
@@ -559,7 +550,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       const int i = t / C::WTL, j = t % C::WTL;
 #pragma unroll
       for (int r = 8 * half; r < 8 * half + 8; r++) {
-        const float sc = R_PER_ROW ? cs[j] * rs[i % RS_SLOTS][r / 4][r % 4] : cs[j];
+        const float sc = R_PER_ROW ? cs[j] * rs[i & 1][r / 4][r % 4] : cs[j];
         acc[i][j][r] = __builtin_fmaf(pr[t % PRB][r], sc, acc[i][j][r]);
       }
     };
@@ -573,17 +564,12 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       constexpr int t = decltype(T)::value;
       constexpr int i = t / C::WTL, j = t % C::WTL;
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (RS_SLOTS == 1 && j == 0) load_rs(i);  // the last fold of the row before is done
-      pr[t % PRB] = mfma_fp8_32x32x64(rf[i % RF_SLOTS][0], lf[j][0], zero);
+      pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][0], lf[j][0], zero);
       __builtin_amdgcn_sched_barrier(0);
       if (D >= 1 && t >= D) fold_half(t - D, 0);
       __builtin_amdgcn_sched_barrier(0);
-      pr[t % PRB] = mfma_fp8_32x32x64(rf[i % RF_SLOTS][1], lf[j][1], pr[t % PRB]);
+      pr[t % PRB] = mfma_fp8_32x32x64(rf[i & 1][1], lf[j][1], pr[t % PRB]);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (RF_SLOTS == 1 && j == C::WTL - 1 && i + 1 < C::WTR) {
-        load_r(i + 1);  // the row's last MFMAs have taken their operands; the fold below covers the reads
-        __builtin_amdgcn_sched_barrier(0);
-      }
       if (D >= 1 && t >= D) fold_half(t - D, 1);
       if (D == 0) {
         fold_half(t, 0);
@@ -591,7 +577,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
       }
       __builtin_amdgcn_sched_barrier(0);
       // the next R row overwrites the fragment and scale slot of row i - 1, whose last fold is done
-      if (RF_SLOTS == 2 && j == 0 && i + 1 < C::WTR) load_r(i + 1);
+      if (j == 0 && i + 1 < C::WTR) load_r(i + 1);
       __builtin_amdgcn_sched_barrier(0);
       // every L fragment has been an MFMA operand by now, so it has left the LDS: the hook (a
       // barrier and the next L loads) costs no extra wait here
@@ -1160,16 +1146,15 @@ static int wgrad_impl(const uint8_t* dyt, const float* sdyt, const uint8_t* xt, 
   p.bias = nullptr; p.bias_dtype = AAMD_NONE; p.bias_group_stride = 0;
   p.goff = group_offsets; p.tile_off = tile_ws;
   // per-row scales on both operands: the 128x128 configuration measured faster for wgrad
-  // (measurement build: tile 1 = 256 x 128, tile 2 = 256 x 256 with wave tiles of 128 x 64)
-  const int cfg = g_opt.tile > 0 ? g_opt.tile : 0;
+  // (measurement build: tile 1 = 256 x 128)
+  const int cfg = g_opt.tile > 0 ? 1 : 0;
   const int BM = cfg ? CfgWgrad::BM : CfgSmall::BM;
-  const int BN = cfg == 2 ? CfgWgrad256::BN : cfg == 1 ? CfgWgrad::BN : CfgSmall::BN;
+  const int BN = cfg ? CfgWgrad::BN : CfgSmall::BN;
   p.Lrows = N; p.Rrows = K; p.nkb = 0; p.E = E; p.nRt = (int)((K + BN - 1) / BN); p.nLt = (int)((N + BM - 1) / BM);
   p.max_kb = (int)(ld_t / kBK);
   p.accumulate = accumulate;
   const int64_t blocks = (int64_t)E * p.nLt * p.nRt;
 #ifdef AAMD_TUNING
-  if (cfg == 2) return launch_gemm<kRaggedK, true, CfgWgrad256>(p, dw_dtype, blocks, st, g_opt);
   if (cfg == 1) return launch_gemm<kRaggedK, true, CfgWgrad>(p, dw_dtype, blocks, st, g_opt);
 #endif
   return launch_gemm<kRaggedK, true, CfgSmall>(p, dw_dtype, blocks, st, g_opt);

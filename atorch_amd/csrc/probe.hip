@@ -29,7 +29,9 @@ __global__ void clock_probe_kernel(unsigned long long* out, long long min_cycles
 // with the fragments of a 128 x 64 wave tile in registers, issue per iteration the sixteen
 // v_mfma_f32_32x32x64_f8f6f4 of one 128-deep step.  FOLD 1: every pair's raw product is folded into the
 // accumulator with sixteen FMAs (the block-scale step); FOLD 2: with sixteen multiplies and sixteen FMAs
-// (per-row scales on both operands, the weight-gradient step); 0: the MFMAs accumulate directly.
+// (per-row scales on both operands, the weight-gradient step); FOLD 3: the accumulator itself is brought to the
+// step's scale with sixteen multiplies that wait for no MFMA of the step, and the MFMAs add to it directly (a
+// measured and rejected form of the block-scale step); 0: the MFMAs accumulate directly.
 template <int FOLD>
 __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(const int* __restrict__ src, float* __restrict__ out,
                                                              int iters, unsigned long long* cyc) {
@@ -57,6 +59,27 @@ __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(const int* __restric
   for (int r = 0; r < 16; r++) rs[r] = 1.0f + 1e-7f * (float)((tid + r) & 7);
   asm volatile("" : "+v"(rs));
   const unsigned long long t0 = __builtin_readcyclecounter();
+  if constexpr (FOLD == 3) {
+    // behind each MFMA of sub-tile t, which adds to its accumulator directly, eight of the sixteen multiplies that
+    // bring the accumulator of sub-tile t + 1 to the step's scale
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        const int i = t >> 1, j = t & 1, ni = ((t + 1) & 7) >> 1, nj = (t + 1) & 1;
+        __builtin_amdgcn_sched_barrier(0);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i][0], lf[j][0], acc[i][j], 0, 0, 0, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 8; r++) acc[ni][nj][r] *= sc;
+        __builtin_amdgcn_sched_barrier(0);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rf[i][1], lf[j][1], acc[i][j], 0, 0, 0, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 8; r < 16; r++) acc[ni][nj][r] *= sc;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  } else
   for (int it = 0; it < iters; it++) {
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -320,7 +343,9 @@ extern "C" int aamd_mfma_probe(const void* operands, int fold, int iters, int wo
   AAMD_REQUIRE(iters >= 1 && iters <= (1 << 20) && workgroups >= 1 && workgroups <= (1 << 16), "mfma_probe: bad sizes");
   AAMD_REQUIRE((reinterpret_cast<uintptr_t>(operands) & 31) == 0, "mfma_probe: operands must be 32-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  if (fold == 2)
+  if (fold == 3)
+    aamd::mfma_probe_kernel<3><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
+  else if (fold == 2)
     aamd::mfma_probe_kernel<2><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);
   else if (fold)
     aamd::mfma_probe_kernel<1><<<workgroups, 512, 0, st>>>((const int*)operands, out, iters, (unsigned long long*)cycles);

@@ -168,7 +168,9 @@ def mfma_probe(kernels, dev, iters=3000):
     cyc = torch.zeros(1, dtype=torch.int64, device=dev)
     res = {}
     for name, ops in sets.items():
-        for fold in (0, 1, 2):  # 1: the block-scale fold (forward, dgrad); 2: per-row scales on both operands (wgrad)
+        # 1: the block-scale fold (forward, dgrad); 2: per-row scales on both operands (wgrad); 3: the accumulator
+        # rescaled instead of a raw product folded (a measured and rejected form of 1)
+        for fold in (0, 1, 2, 3):
             st = torch.cuda.current_stream().cuda_stream
             check(lib().aamd_mfma_probe(ops.data_ptr(), fold, iters, wgs, out.data_ptr(), cyc.data_ptr(), st))
             torch.cuda.synchronize()
@@ -179,7 +181,7 @@ def mfma_probe(kernels, dev, iters=3000):
             torch.cuda.synchronize()
             ms = a.elapsed_time(b)
             fl = wgs * 8 * iters * 16 * 131072.0
-            key = name + ("", "+fold", "+fold_per_row")[fold]
+            key = name + ("", "+fold", "+fold_per_row", "+rescaled_accumulator")[fold]
             res[key] = {"TFLOP/s": round(fl / ms / 1e9, 1)}
             if fold:
                 # with the fold the two waves of a SIMD alternate on its pipe, so the probed wave runs for the

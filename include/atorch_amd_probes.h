@@ -23,7 +23,7 @@ const char *aamd_probes_last_error(void);
  * The grouped GEMMs of the product library (same kernels, same arguments as aamd_grouped_gemm_fp8_nt and
  * aamd_grouped_gemm_fp8_wgrad) with the launch choices the library otherwise makes by itself pinned for
  * this one call: opts = {tile, group_r, gl, ls_batch}, each -1 for the library's own choice.
- *   tile: 0 = 128x128 tiles, 1 = the large configuration (wgrad: 1 = 256x128, 2 = 256x256 tiles);
+ *   tile: 0 = 128x128 tiles, 1 = the large configuration (wgrad: 256x128 tiles);
  *   group_r: the tile order groups R tiles (1) or L tiles (0); gl: tiles sharing a panel in the tile order;
  *   ls_batch: 0 = scales fetched one contraction block at a time (which the 128x128 tiles do: the large
  *   configuration of the block-scaled GEMM takes its scales in batches only and is then not chosen).
@@ -51,7 +51,8 @@ int aamd_clock_probe(uint64_t *out, int64_t min_cycles, void *stream);
  * limit): `workgroups` workgroups of eight waves issue, `iters` times, the sixteen
  * v_mfma_f32_32x32x64_f8f6f4 of one 128-deep step of a 128 x 64 wave tile, with the block-scale fold
  * (16 FMAs per MFMA pair) when fold == 1, or the fold of per-row scales on both operands (16 multiplies and 16 FMAs
- * per MFMA pair, the weight-gradient step) when fold == 2.  FLOP = workgroups * 8 * iters * 16 * 131072.
+ * per MFMA pair, the weight-gradient step) when fold == 2; fold == 3: sixteen multiplies per pair rescale the accumulator
+ * the MFMAs then add to directly (no raw-product buffer, no wait for an MFMA result).  FLOP = workgroups * 8 * iters * 16 * 131072.
  *   operands: 64 * 512 * 12 * 32 bytes of fp8 codes (any values), 32-byte aligned
  *   out: workgroups * 512 floats (checksums); cycles[0]: shader cycles one wave spent in the loop.
  */

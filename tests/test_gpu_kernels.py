@@ -532,7 +532,7 @@ def test_grouped_gemm_nt_scale_batches_of_the_large_tiles(dev, K):
     assert rel_err(y.cpu(), ref.float().cpu()) <= GEMM_TOL_F32
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2], ids=["128x128", "256x128", "256x256"])
+@pytest.mark.parametrize("tile", [0, 1], ids=["128x128", "256x128"])
 def test_grouped_gemm_wgrad_pinned_tile_configurations(dev, tile):
     """The tile configurations of the weight-gradient GEMM (the product library runs the first; the others are
     measurement builds) on ragged
