@@ -183,10 +183,13 @@ def mfma_probe(kernels, dev, iters=3000):
             fl = wgs * 8 * iters * 16 * 131072.0
             key = name + ("", "+fold", "+fold_per_row", "+rescaled_accumulator")[fold]
             res[key] = {"TFLOP/s": round(fl / ms / 1e9, 1)}
-            if fold:
+            if fold in (1, 2):
                 # with the fold the two waves of a SIMD alternate on its pipe, so the probed wave runs for the
                 # whole of its round (one of wgs/256): its cycle count over that time is the shader clock
                 res[key]["sclk_ghz"] = round(int(cyc.item()) / (ms * 1e6 / (wgs / 256)), 3)
+            if fold == 1:
+                res[key]["board_power"] = power_under(
+                    lambda: check(lib().aamd_mfma_probe(ops.data_ptr(), 1, iters, wgs, out.data_ptr(), cyc.data_ptr(), st)), 1.0)
     return res
 
 
@@ -264,6 +267,71 @@ def host_threads():
     n = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(n)
     return n
+
+
+class PowerSampler:
+    """Board power (W) while a region runs, read from the amdgpu hwmon file every 25 ms by a thread of this
+    process; the package power cap is read beside it.  The grouped GEMMs of the benchmark run at that cap:
+    their clock, and with it their throughput, is what the power management leaves them."""
+
+    def __init__(self):
+        import glob
+
+        hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.file = next((os.path.join(h, n) for h in hw for n in ("power1_input", "power1_average")
+                          if os.path.exists(os.path.join(h, n))), None)  # fmt: skip
+        self.cap = None
+        for h in hw:
+            try:
+                self.cap = int(open(os.path.join(h, "power1_cap")).read()) / 1e6
+                break
+            except (OSError, ValueError):
+                pass
+        self.vals = []
+
+    def __enter__(self):
+        import threading
+
+        self._stop = False
+
+        def poll():
+            while not self._stop and self.file:
+                try:
+                    self.vals.append(int(open(self.file).read()) / 1e6)
+                except (OSError, ValueError):
+                    return
+                time.sleep(0.025)
+
+        self._t = threading.Thread(target=poll, daemon=True)
+        self._t.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        self._t.join()
+        return False
+
+    def summary(self):
+        if not self.vals:
+            return None
+        v = self.vals[len(self.vals) // 4 :] or self.vals  # the first samples still see the ramp
+        return {"mean_W": round(sum(v) / len(v), 1), "max_W": round(max(v), 1), "cap_W": self.cap, "samples": len(v)}
+
+
+def power_under(fn, seconds=1.5):
+    """Board power while fn() is launched back to back for `seconds`."""
+    ps = PowerSampler()
+    if ps.file is None:
+        return None
+    fn()
+    torch.cuda.synchronize()
+    with ps:
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+    return ps.summary()
 
 
 class Timer:
@@ -426,6 +494,9 @@ def run_gemm(args, kernels, dev, workload=None, steps=None, warmup=None, cpu_bas
               "empty_groups": int((counts == 0).sum()), "operands": args.operands}
     if probes:
         extras["sclk_ghz_under_forward_gemm"] = clock_under(lambda: layers[0].fwd(kernels), dev)
+        extras["board_power_under_forward_gemm"] = power_under(lambda: layers[0].fwd(kernels))
+        if backward:
+            extras["board_power_under_wgrad_gemm"] = power_under(lambda: layers[0].wgrad(kernels))
     if backward:
         wg_avg = wg_timer.mean()
         wg_flops = sum(L.flops for L in layers) / len(layers)
@@ -519,7 +590,7 @@ def operand_data_probe(kernels, layer, dev, iters=5):
         ms = a.elapsed_time(b) / iters
         tf = layer.flops / ms / 1e9
         res[name] = {"TFLOP/s": round(tf, 1), "frac": round(tf / PEAK_FP8_TFLOPS, 4), "avg_launch_ms": round(ms, 4),
-                     "sclk_ghz": clock_under(fn, dev)}  # fmt: skip
+                     "sclk_ghz": clock_under(fn, dev), "board_power": power_under(fn, 1.0)}  # fmt: skip
     del zx, zw, out
     return res
 
