@@ -306,6 +306,59 @@ def test_moe_layer_matches_composition_and_float_reference(dev, use_swiglu):
         Grouped_GEMM_MoE(H, F, 0.0, E, k, use_expert_parallelism=True)
 
 
+@pytest.mark.parametrize("variant", ["separate_kn", "bias_gelu", "bias_swiglu_megablocks"])
+def test_moe_layer_other_parameterisations(dev, variant):
+    """Separate gate / up weights stored [E, H, F] (merge_w1_v1=False, transpose_w1=False), and use_bias with both
+    activations: the layer equals permute -> grouped_mlp with the same parameters -> combine, bit for bit, gradients of
+    every parameter included."""
+    from atorch_amd.expert_mlp import grouped_mlp
+    from atorch_amd.moe_layer import Grouped_GEMM_MoE
+    from atorch_amd.token_dispatcher import MoETokenDispatcher
+
+    T, H, F, E, k = 160, 256, 128, 4, 2
+    torch.manual_seed(2)
+    kw = {"device": dev, "dtype": torch.bfloat16}
+    if variant == "separate_kn":
+        layer = Grouped_GEMM_MoE(H, F, 0.0, E, k, use_swiglu=True, merge_w1_v1=False, transpose_w1=False, **kw)
+        assert layer.w1.shape == (E, H, F) and layer.v1.shape == (E, H, F) and layer.has_v1()
+    elif variant == "bias_gelu":
+        layer = Grouped_GEMM_MoE(H, F, 0.0, E, k, use_swiglu=False, use_bias=True, implementation_type="Megatron", **kw)
+    else:
+        layer = Grouped_GEMM_MoE(H, F, 0.0, E, k, use_swiglu=True, use_bias=True, implementation_type="MegaBlocks", **kw)
+    if layer.use_bias:
+        with torch.no_grad():
+            layer.b1.copy_(randn_bf16(tuple(layer.b1.shape), 11, std=0.5))
+            layer.b2.copy_(randn_bf16(tuple(layer.b2.shape), 12, std=0.5))
+    params = [p for p in layer.parameters()]
+    x = randn_bf16((T, H), 13)
+    idx, probs = topk_routing(T, E, k, seed=14, zipf_s=1.0)
+    probs = probs.bfloat16()
+    dout = randn_bf16((T, H), 15, std=1e-2).to(dev)
+
+    xg = x.to(dev).requires_grad_(True)
+    out = layer(xg, probs.to(dev), idx.to(dev))
+    out.backward(dout)
+    got = [out.detach().clone(), xg.grad.clone()] + [p.grad.clone() for p in params]
+    layer.zero_grad()
+
+    d = MoETokenDispatcher(E, k)
+    xg2 = x.to(dev).requires_grad_(True)
+    permuted, goff = d.token_permutation(xg2, probs.to(dev), idx.to(dev))
+    y = grouped_mlp(permuted, layer.w1, layer.w2, goff[1:] - goff[:-1], v1=layer.v1 if layer.has_v1() else None,
+                    b1=layer.b1 if layer.use_bias else None, b2=layer.b2 if layer.use_bias else None,
+                    activation="swiglu" if layer.use_swiglu else "gelu", transpose_w1=layer.transpose_w1)  # fmt: skip
+    out2, _ = d.token_unpermutation(y)
+    out2.backward(dout)
+    want = [out2.detach(), xg2.grad] + [p.grad for p in params]
+    assert len(got) == len(want) and all(g is not None for g in want)
+    for i, (a, b) in enumerate(zip(got, want)):
+        if layer.use_bias and a.shape in (tuple(layer.b1.shape), tuple(layer.b2.shape)):
+            torch.testing.assert_close(a.float(), b.float(), rtol=2e-2, atol=1e-4)  # atomics: order of an fp32 sum
+        else:
+            assert torch.equal(a, b), f"tensor {i} differs from the composition"
+    assert float(out.detach().float().abs().max()) > 0
+
+
 @pytest.mark.filterwarnings("ignore:The AccumulateGrad node")
 def test_moe_layer_training_step_replays_from_one_graph(dev):
     """Forward and backward of the whole layer (router preprocess, fused permute + quantise, six grouped GEMMs, the
