@@ -158,6 +158,47 @@ def test_dual_grouped_quant_full_size(oracle, dev):
         assert bool((q_t[:, pad[e] + m : pad[e + 1]].view(torch.uint8) == 0).all())
 
 
+@pytest.mark.parametrize("T,E,k,H,heavy", [(65536, 64, 8, 7168, True), (32768, 60, 4, 2048, False)],
+                         ids=["c5_shape", "c4_shape"])
+def test_permute_quant_dual_grouped_full_size(oracle, dev, T, E, k, H, heavy):
+    """The training form of the fused permute at the sizes of the quant / permute configuration (65536 x 7168, top-8
+    into 64 experts) and of the Qwen-like one: equal to permute_rows followed by the dual grouped quantiser bit for
+    bit over the whole outputs, its row-wise part equal to the scatter form (every token quantised once), and sampled
+    columns of sampled groups against the oracle."""
+    from atorch_amd import kernels as K
+
+    x = _student_t((T, H), dev, seed=0) if heavy else _randn((T, H), dev, 1.0, 7)
+    idx, _ = _routing(T, E, k, dev)
+    sorted_idx, row_map, goff = K.moe_preprocess(idx, E)
+    M = T * k
+    q, s, q_t, s_t = K.permute_tile_quant_dual_grouped(x, sorted_idx, k, goff, E)
+    counts = (goff[1:] - goff[:-1]).cpu().tolist()
+    pad = [0]
+    for c in counts:
+        pad.append(pad[-1] + (c + TILE - 1) // TILE * TILE)
+    pe = pad[-1]
+    # row-wise part: the codes and scales of the scatter form
+    q1, s1 = K.permute_tile_quant(x, row_map, k, M)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s, s1)
+    del q1, s1
+    # everything: the two separate kernels
+    xp = K.permute_rows(x, row_map, k, M)
+    q2, s2, q_t2, s_t2 = K.tile_quant_dual_grouped(xp, goff, E, ld_t=q_t.shape[1])
+    assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+    assert torch.equal(q_t.view(torch.uint8)[:, :pe], q_t2.view(torch.uint8)[:, :pe])
+    assert torch.equal(s_t[: pe // TILE], s_t2[: pe // TILE])
+    del q2, s2, q_t2, s_t2
+    # sampled groups against the oracle (256 columns keep the CPU work small)
+    offs = goff.cpu().tolist()
+    for e in (0, E // 3, E - 1):
+        m = counts[e]
+        xe = xp[offs[e] : offs[e] + m, :256].cpu()
+        qt_o, st_o = oracle.tile_quant_t_grouped(xe, [m])
+        assert torch.equal(q_t[:256, pad[e] : pad[e + 1]].view(torch.uint8).cpu(), qt_o[:, : pad[e + 1] - pad[e]])
+        assert torch.equal(s_t[pad[e] // TILE : pad[e + 1] // TILE, :256].cpu(), st_o[: (pad[e + 1] - pad[e]) // TILE])
+        assert bool((q_t[:, pad[e] + m : pad[e + 1]].view(torch.uint8) == 0).all())
+
+
 # ------------------------------------------------------------------------------------------
 # grouped GEMMs at full size
 # ------------------------------------------------------------------------------------------
