@@ -494,9 +494,10 @@ def run_gemm(args, kernels, dev, workload=None, steps=None, warmup=None, cpu_bas
               "empty_groups": int((counts == 0).sum()), "operands": args.operands}
     if probes:
         extras["sclk_ghz_under_forward_gemm"] = clock_under(lambda: layers[0].fwd(kernels), dev)
-        extras["board_power_under_forward_gemm"] = power_under(lambda: layers[0].fwd(kernels))
-        if backward:
-            extras["board_power_under_wgrad_gemm"] = power_under(lambda: layers[0].wgrad(kernels))
+        if not args.no_extras:
+            extras["board_power_under_forward_gemm"] = power_under(lambda: layers[0].fwd(kernels))
+            if backward:
+                extras["board_power_under_wgrad_gemm"] = power_under(lambda: layers[0].wgrad(kernels))
     if backward:
         wg_avg = wg_timer.mean()
         wg_flops = sum(L.flops for L in layers) / len(layers)
