@@ -13,7 +13,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libatorch_amd_fp8.so")
 
 OK, ERR_ARG, ERR_HIP = 0, 1, 2
 NONE, BF16, F32, F16 = -1, 0, 1, 2
-ABI_VERSION = 3
+QT_ROWS, QT_BLOCKED = 0, 1  # layouts of the transposed codes
+ABI_VERSION = 4
 
 _lib: Optional[ctypes.CDLL] = None
 
@@ -28,25 +29,25 @@ SIGNATURES = {
     "aamd_permute_rows": (_int, [_vp, _int, _i64, _i64, _vp, _int, _i64, _vp, _vp]),
     "aamd_quant_1x128_dual_grouped": (
         _int,
-        [_vp, _int, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _f32, _vp],
+        [_vp, _int, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp],
     ),
     "aamd_permute_quant_1x128_dual_grouped": (
         _int,
-        [_vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _f32, _vp],
+        [_vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp],
     ),
     "aamd_swiglu_quant_1x128": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     "aamd_swiglu_quant_1x128_dual_grouped": (
         _int,
-        [_vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+        [_vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp],
     ),
     "aamd_swiglu_bwd_quant_1x128_dual_grouped": (
         _int,
-        [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+        [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp],
     ),
     "aamd_gelu_quant_1x128": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     "aamd_gelu_quant_1x128_dual_grouped": (
         _int,
-        [_vp, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+        [_vp, _vp, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp],
     ),
     "aamd_bias_gather_add": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
     "aamd_bias_gather_add_bgrad": (_int, [_vp, _vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
@@ -58,7 +59,7 @@ SIGNATURES = {
     ),
     "aamd_grouped_gemm_fp8_wgrad": (
         _int,
-        [_vp, _vp, _vp, _vp, _i64, _vp, _int, _vp, _i64, _i64, _vp, _int, _i64, _int, _vp],
+        [_vp, _vp, _vp, _vp, _i64, _int, _vp, _int, _vp, _i64, _i64, _vp, _int, _i64, _int, _vp],
     ),
     "aamd_grouped_gemm_fp8_nt_static": (
         _int,

@@ -19,7 +19,7 @@ SIGNATURES = {
     ),
     "aamd_tuning_grouped_gemm_fp8_wgrad": (
         _int,
-        [_vp, _vp, _vp, _vp, _i64, _vp, _int, _vp, _i64, _i64, _vp, _int, _i64, _int, _opts, _vp],
+        [_vp, _vp, _vp, _vp, _i64, _int, _vp, _int, _vp, _i64, _i64, _vp, _int, _i64, _int, _opts, _vp],
     ),
     "aamd_clock_probe": (_int, [_vp, _i64, _vp]),
     "aamd_stream_probe": (_int, [_vp, _vp, _int, _int, _i64, _i64, _vp]),

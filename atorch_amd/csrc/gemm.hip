@@ -57,6 +57,7 @@ struct GemmParams {
   const int64_t* goff;      // [E+1] rows per group prefix (device); nullptr: one group [0, Lrows)
   const int32_t* tile_off;  // [E+1] tile prefix (device)
   int64_t ldl, ldr;                          // row strides of L and R (bytes)
+  int64_t l_kb_stride, r_kb_stride;          // bytes between consecutive 128-wide contraction blocks of a row
   int64_t r_group_stride;                    // bytes between the R matrices of consecutive groups
   int64_t ls_row_stride, ls_blk_stride;      // L scale (row, block) strides, floats
   int64_t rs_row_stride, rs_blk_stride, rs_group_stride;
@@ -303,8 +304,8 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   const int rvalid = rleft < BN ? (int)rleft : BN;  // a multiple of 128
 
   // uniform tile bases + per-thread 32-bit offsets
-  const uint8_t* Lbase = p.L + uniform_i64(l0 * p.ldl + (int64_t)kb0 * kBK);
-  const uint8_t* Rbase = p.R + uniform_i64((int64_t)g * p.r_group_stride + r0 * p.ldr + (int64_t)kb0 * kBK);
+  const uint8_t* Lbase = p.L + uniform_i64(l0 * p.ldl + (int64_t)kb0 * p.l_kb_stride);
+  const uint8_t* Rbase = p.R + uniform_i64((int64_t)g * p.r_group_stride + r0 * p.ldr + (int64_t)kb0 * p.r_kb_stride);
   const float* Lsg = p.Ls + (int64_t)kb0 * p.ls_blk_stride;
   const float* Rsg = p.Rs + (int64_t)g * p.rs_group_stride + (int64_t)kb0 * p.rs_blk_stride;
 
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
   // One wave instruction of the L (R) tile of a step; the last one of a half also carries that
   // half's scale loads.  L half: the L tile and, from the waves that own them, the L scales.
   auto dmaL_tile = [&](int n, int kb, uint8_t* Ld) {
-    const uint8_t* lb = Lbase + (int64_t)kb * kBK;
+    const uint8_t* lb = Lbase + (int64_t)kb * p.l_kb_stride;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  ::"v"(ltail[n] ? voffLt : voffL), "s"(lb + lslab[n]),
                    "s"(lds_addr(Ld) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(C::NT, C::NT == 256 ? 2 : 1) void grouped_gemm_kern
     if (l_side && step_scale) dma_scale(kb, Sd);
   };
   auto dmaR_tile = [&](int n, int kb, uint8_t* Rd) {
-    const uint8_t* rb = Rbase + (int64_t)kb * kBK;
+    const uint8_t* rb = Rbase + (int64_t)kb * p.r_kb_stride;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  ::"v"(voffR), "s"(rb + rslab[n]),
                    "s"(lds_addr(Rd) + (uint32_t)((wave * 8 + (NT / 8) * n) * kBK))
@@ -1049,6 +1050,7 @@ static int gemm_nt_impl(const uint8_t* a, int64_t lda, const float* a_s, const u
   }
   GemmParams p = {};
   p.L = a; p.ldl = lda; p.Ls = a_s; p.ls_row_stride = K / kBK; p.ls_blk_stride = 1;
+  p.l_kb_stride = p.r_kb_stride = kBK;
   // 1: batches by 16-byte loads; 2 (256x256 configuration only): by 4-byte loads
   p.ls_batch = large && !b_tile_scaled ? (batches16 && aligned16(b_s) ? 1 : 2) : (batches16 ? 1 : 0);
   p.R = b; p.ldr = K; p.r_group_stride = N * K;
@@ -1122,7 +1124,7 @@ extern "C" int aamd_grouped_gemm_fp8_nt_static(const uint8_t* a, int64_t lda, co
 #endif  // !AAMD_TUNING
 
 static int wgrad_impl(const uint8_t* dyt, const float* sdyt, const uint8_t* xt, const float* sxt, int64_t ld_t,
-                      const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t N, int64_t K, void* dw,
+                      int q_t_layout, const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t N, int64_t K, void* dw,
                       int dw_dtype, int64_t expert_stride, int accumulate, void* stream,
                       const GemmOptions& g_opt = GemmOptions()) {
   AAMD_REQUIRE(dw_dtype == AAMD_BF16 || dw_dtype == AAMD_F32, "grouped_gemm_wgrad: unsupported output dtype %d", dw_dtype);
@@ -1131,6 +1133,7 @@ static int wgrad_impl(const uint8_t* dyt, const float* sdyt, const uint8_t* xt, 
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "grouped_gemm_wgrad: group_offsets / tile_ws required");
   AAMD_REQUIRE(ld_t >= 0 && ld_t % kBK == 0, "grouped_gemm_wgrad: ld_t=%lld must be a multiple of 128", (long long)ld_t);
   AAMD_REQUIRE(ld_t < (1LL << 23), "grouped_gemm_wgrad: ld_t too large");
+  AAMD_REQUIRE(q_t_layout == AAMD_QT_ROWS || q_t_layout == AAMD_QT_BLOCKED, "grouped_gemm_wgrad: unknown operand layout %d", q_t_layout);
   if (N == 0 || K == 0) return AAMD_OK;
   AAMD_REQUIRE(dw && (ld_t == 0 || (dyt && sdyt && xt && sxt)), "grouped_gemm_wgrad: null pointer");
   AAMD_REQUIRE(aligned16(dyt) && aligned16(xt) && aligned16(dw), "grouped_gemm_wgrad: pointers must be 16-byte aligned");
@@ -1139,8 +1142,15 @@ static int wgrad_impl(const uint8_t* dyt, const float* sdyt, const uint8_t* xt, 
   int rc = launch_group_tile_offsets(group_offsets, E, kBK, tile_ws, st);
   if (rc) return rc;
   GemmParams p = {};
-  p.L = dyt; p.ldl = ld_t; p.Ls = sdyt; p.ls_row_stride = 1; p.ls_blk_stride = N;
-  p.R = xt; p.ldr = ld_t; p.r_group_stride = 0;
+  p.L = dyt; p.Ls = sdyt; p.ls_row_stride = 1; p.ls_blk_stride = N;
+  p.R = xt; p.r_group_stride = 0;
+  if (q_t_layout == AAMD_QT_BLOCKED) {  // [ld_t / 128, rows, 128]: a contraction block of all rows is one slab
+    p.ldl = p.ldr = kBK;
+    p.l_kb_stride = N * kBK; p.r_kb_stride = K * kBK;
+  } else {
+    p.ldl = p.ldr = ld_t;
+    p.l_kb_stride = p.r_kb_stride = kBK;
+  }
   p.Rs = sxt; p.rs_row_stride = 1; p.rs_blk_stride = K; p.rs_group_stride = 0;
   p.C = dw; p.ldc = K; p.c_group_stride = expert_stride;
   p.bias = nullptr; p.bias_dtype = AAMD_NONE; p.bias_group_stride = 0;
@@ -1162,10 +1172,11 @@ static int wgrad_impl(const uint8_t* dyt, const float* sdyt, const uint8_t* xt, 
 
 #ifndef AAMD_TUNING
 extern "C" int aamd_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt, const uint8_t* xt,
-                                           const float* sxt, int64_t ld_t, const int64_t* group_offsets, int E,
-                                           int32_t* tile_ws, int64_t N, int64_t K, void* dw, int dw_dtype,
-                                           int64_t expert_stride, int accumulate, void* stream) {
-  return wgrad_impl(dyt, sdyt, xt, sxt, ld_t, group_offsets, E, tile_ws, N, K, dw, dw_dtype, expert_stride, accumulate,
+                                           const float* sxt, int64_t ld_t, int q_t_layout,
+                                           const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t N,
+                                           int64_t K, void* dw, int dw_dtype, int64_t expert_stride, int accumulate,
+                                           void* stream) {
+  return wgrad_impl(dyt, sdyt, xt, sxt, ld_t, q_t_layout, group_offsets, E, tile_ws, N, K, dw, dw_dtype, expert_stride, accumulate,
                     stream);
 }
 #else
@@ -1183,14 +1194,14 @@ extern "C" int aamd_tuning_grouped_gemm_fp8_nt(const uint8_t* a, int64_t lda, co
                       bias_dtype, stream, o);
 }
 extern "C" int aamd_tuning_grouped_gemm_fp8_wgrad(const uint8_t* dyt, const float* sdyt, const uint8_t* xt,
-                                                  const float* sxt, int64_t ld_t, const int64_t* group_offsets, int E,
-                                                  int32_t* tile_ws, int64_t N, int64_t K, void* dw, int dw_dtype,
-                                                  int64_t expert_stride, int accumulate, const int* opts,
-                                                  void* stream) {
+                                                  const float* sxt, int64_t ld_t, int q_t_layout,
+                                                  const int64_t* group_offsets, int E, int32_t* tile_ws, int64_t N,
+                                                  int64_t K, void* dw, int dw_dtype, int64_t expert_stride,
+                                                  int accumulate, const int* opts, void* stream) {
   AAMD_REQUIRE(opts != nullptr, "tuning_grouped_gemm_wgrad: null options");
   GemmOptions o;
   o.tile = opts[0]; o.group_r = opts[1]; o.gl = opts[2]; o.ls_batch = opts[3];
-  return wgrad_impl(dyt, sdyt, xt, sxt, ld_t, group_offsets, E, tile_ws, N, K, dw, dw_dtype, expert_stride, accumulate,
-                    stream, o);
+  return wgrad_impl(dyt, sdyt, xt, sxt, ld_t, q_t_layout, group_offsets, E, tile_ws, N, K, dw, dw_dtype, expert_stride,
+                    accumulate, stream, o);
 }
 #endif

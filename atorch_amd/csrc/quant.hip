@@ -305,6 +305,16 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
   }
 }
 
+// Where tile (token tile pt, column tile kc) of the transposed codes goes, and the stride of its 128 rows.
+// Layout 0: q_t is [cols, ld_t], a row per column of x; layout 1 (AAMD_QT_BLOCKED): q_t is [ld_t / 128, cols, 128],
+// token-block-major, so that a tile is 16 KB of consecutive bytes and the tiles of a token block follow each other:
+// the kernel then writes the transposed codes as one sequential sweep instead of 128-byte pieces ld_t apart.
+__device__ __forceinline__ uint8_t* qt_tile(uint8_t* q_t, int blocked, int64_t cols, uint32_t ld_t, int pt, int kc, uint32_t* ld) {
+  *ld = blocked ? (uint32_t)kTile : ld_t;
+  return blocked ? q_t + ((int64_t)pt * cols + (int64_t)kc * kTile) * kTile
+                 : q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile;
+}
+
 // One 128 x 128 tile of the dual quantiser: token tile pt of group g, column tile kc.  Everything that
 // locates the tile is the same in every lane, so each access is a scalar base plus a 32-bit lane offset
 // (the launchers bound the row strides so that 128 rows stay below 2^32 bytes).
@@ -313,9 +323,9 @@ __device__ __forceinline__ void store_staged_tile(const uint8_t* tile_t, uint8_t
 template <typename IN, bool FULL, bool GATHER = false>
 __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ x, uint32_t ldx, int nt, int64_t m0,
                                           int mvalid, int pt, int kc, uint8_t* __restrict__ q, float* __restrict__ s,
-                                          uint8_t* __restrict__ q_t, float* __restrict__ s_t, uint32_t ld_t, float eps,
-                                          int64_t gate_off, u16* __restrict__ h_out, uint8_t* tile_t, Divider* cdiv,
-                                          const uint32_t* src_row = nullptr) {
+                                          uint8_t* __restrict__ q_t, float* __restrict__ s_t, uint32_t ld_t, int blocked,
+                                          float eps, int64_t gate_off, u16* __restrict__ h_out, uint8_t* tile_t,
+                                          Divider* cdiv, const uint32_t* src_row = nullptr) {
   const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
   const int64_t cols = (int64_t)nt * kTile;
@@ -409,14 +419,16 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
     }
     *reinterpret_cast<v2i*>(tile_t + staged_off(c * 8 + j, gr * 8)) = quant8(col, cdiv[j * 16 + c]);
   }
-  store_staged_tile(tile_t, q_t + (int64_t)kc * kTile * ld_t + (int64_t)pt * kTile, ld_t);
+  uint32_t ld_out;
+  uint8_t* const out_t = qt_tile(q_t, blocked, cols, ld_t, pt, kc, &ld_out);
+  store_staged_tile(tile_t, out_t, ld_out);
 }
 
 template <typename IN>
 __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ goff,
     const int32_t* __restrict__ tile_off, int E, uint8_t* __restrict__ q, float* __restrict__ s,
-    uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, float eps, int64_t gate_off,
+    uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t, int blocked, float eps, int64_t gate_off,
     u16* __restrict__ h_out) {
   // the per-row-group column maxima are dead before the transposed codes are staged: one region
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
@@ -445,9 +457,9 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   const int64_t left = goff[g + 1] - m0;
   const int mvalid = left < kTile ? (int)left : kTile;
   if (mvalid == kTile)
-    dual_tile<IN, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, gate_off, h_out, tile_t, cdiv);
+    dual_tile<IN, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, gate_off, h_out, tile_t, cdiv);
   else
-    dual_tile<IN, false>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, gate_off, h_out, tile_t, cdiv);
+    dual_tile<IN, false>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, gate_off, h_out, tile_t, cdiv);
 }
 
 // The dual quantiser with the token permute fused in: x holds the tokens in their original order, and permuted
@@ -461,7 +473,7 @@ __global__ __launch_bounds__(256) void quant_dual_gather_kernel(
     const typename IN::elem* __restrict__ x, int64_t ldx, int nt, const int64_t* __restrict__ sorted_idx,
     uint32_t magic, int sh, uint32_t T, const int64_t* __restrict__ goff, const int32_t* __restrict__ tile_off, int E,
     uint8_t* __restrict__ q, float* __restrict__ s, uint8_t* __restrict__ q_t, float* __restrict__ s_t, int64_t ld_t,
-    float eps) {
+    int blocked, float eps) {
   __shared__ __attribute__((aligned(16))) uint8_t tile_t[kTile * kTLd];
   __shared__ Divider cdiv[kTile];
   __shared__ uint32_t src_row[kTile];
@@ -489,9 +501,9 @@ __global__ __launch_bounds__(256) void quant_dual_gather_kernel(
   }
   __syncthreads();
   if (mvalid == kTile)
-    dual_tile<IN, true, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, 0, nullptr, tile_t, cdiv, src_row);
+    dual_tile<IN, true, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, 0, nullptr, tile_t, cdiv, src_row);
   else
-    dual_tile<IN, false, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, eps, 0, nullptr, tile_t, cdiv, src_row);
+    dual_tile<IN, false, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, 0, nullptr, tile_t, cdiv, src_row);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -520,8 +532,9 @@ __device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa 
                                                      int64_t gate_off, const u16* __restrict__ xd, uint32_t ld_dh, int nt,
                                                      int64_t m0, int mvalid, int pt, int f, uint8_t* __restrict__ q,
                                                      float* __restrict__ s, uint8_t* __restrict__ q_t,
-                                                     float* __restrict__ s_t, uint32_t ld_t, u16* __restrict__ g_out,
-                                                     uint8_t (*tile_t)[kTile * kTLd], Divider (*cdiv)[kTile]) {
+                                                     float* __restrict__ s_t, uint32_t ld_t, int blocked,
+                                                     u16* __restrict__ g_out, uint8_t (*tile_t)[kTile * kTLd],
+                                                     Divider (*cdiv)[kTile]) {
   const int tid = threadIdx.x, gr = tid >> 4, c = tid & 15;
   const int half = nt / 2;
   const int64_t cols = (int64_t)nt * kTile;
@@ -627,12 +640,13 @@ __device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa 
   __syncthreads();
 #pragma unroll
   for (int w = 0; w < 2; w++) {
-    uint8_t* const out = q_t + (int64_t)(w == 0 ? f : half + f) * kTile * ld_t + (int64_t)pt * kTile;
+    uint32_t ld_out;
+    uint8_t* const out = qt_tile(q_t, blocked, cols, ld_t, pt, w == 0 ? f : half + f, &ld_out);
 #pragma unroll
     for (int n = 0; n < 2; n++) {
       const int idx = tid + 512 * n;
       const int r = idx >> 3, ch = idx & 7;
-      st_nt(out, (uint32_t)r * ld_t + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(&tile_t[w][staged_off(r, ch * 16)]));
+      st_nt(out, (uint32_t)r * ld_out + (uint32_t)ch * 16, *reinterpret_cast<const v4i*>(&tile_t[w][staged_off(r, ch * 16)]));
     }
   }
 }
@@ -643,7 +657,7 @@ __global__ __launch_bounds__(512, 4) void swiglu_bwd_dual_kernel(const u16* __re
                                                               const int32_t* __restrict__ tile_off, int E,
                                                               uint8_t* __restrict__ q, float* __restrict__ s,
                                                               uint8_t* __restrict__ q_t, float* __restrict__ s_t,
-                                                              int64_t ld_t, u16* __restrict__ g_out) {
+                                                              int64_t ld_t, int blocked, u16* __restrict__ g_out) {
   __shared__ __attribute__((aligned(16))) uint8_t tile_ts[2][kTile * kTLd];
   __shared__ Divider cdivs[2][kTile];
   __shared__ int slot;
@@ -669,10 +683,10 @@ __global__ __launch_bounds__(512, 4) void swiglu_bwd_dual_kernel(const u16* __re
   const u16* const xd = dh + m0 * ld_dh + (int64_t)f * kTile;
   if (mvalid == kTile)
     swiglu_bwd_dual_tile<true>(xa, (uint32_t)ld, gate_off, xd, (uint32_t)ld_dh, nt, m0, mvalid, pt, f, q, s, q_t, s_t,
-                               (uint32_t)ld_t, g_out, tile_ts, cdivs);
+                               (uint32_t)ld_t, blocked, g_out, tile_ts, cdivs);
   else
     swiglu_bwd_dual_tile<false>(xa, (uint32_t)ld, gate_off, xd, (uint32_t)ld_dh, nt, m0, mvalid, pt, f, q, s, q_t, s_t,
-                                (uint32_t)ld_t, g_out, tile_ts, cdivs);
+                                (uint32_t)ld_t, blocked, g_out, tile_ts, cdivs);
 }
 
 // The 8x8 byte matrix held as eight rows of two dwords, transposed with byte permutes: cols[j]
@@ -835,9 +849,10 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
 
 extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t M, int64_t cols, int64_t ldx,
                                              const int64_t* group_offsets, int E, int32_t* tile_ws, uint8_t* q,
-                                             float* s, uint8_t* q_t, float* s_t, int64_t ld_t, float eps,
-                                             void* stream) {
+                                             float* s, uint8_t* q_t, float* s_t, int64_t ld_t, int q_t_layout,
+                                             float eps, void* stream) {
   AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "quant_dual: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(q_t_layout == AAMD_QT_ROWS || q_t_layout == AAMD_QT_BLOCKED, "quant_dual: unknown q_t layout %d", q_t_layout);
   AAMD_REQUIRE(M >= 0 && cols >= 0 && cols % kTile == 0, "quant_dual: cols=%lld must be a multiple of 128",
                (long long)cols);
   AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0 && ldx < kMaxTileLd, "quant_dual: bad ldx=%lld", (long long)ldx);
@@ -861,11 +876,11 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
   dim3 grid((unsigned)(cols / kTile), (unsigned)grid_tiles), block(256);
   const int nt = (int)(cols / kTile);
   if (x_dtype == AAMD_BF16)
-    quant_dual_grouped_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
+    quant_dual_grouped_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, q_t_layout, eps, 0, nullptr);
   else if (x_dtype == AAMD_F16)
-    quant_dual_grouped_kernel<F16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
+    quant_dual_grouped_kernel<F16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, q_t_layout, eps, 0, nullptr);
   else
-    quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps, 0, nullptr);
+    quant_dual_grouped_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, q_t_layout, eps, 0, nullptr);
   AAMD_LAUNCH_CHECK("quant_dual_grouped");
   return AAMD_OK;
 }
@@ -873,9 +888,10 @@ extern "C" int aamd_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t
 extern "C" int aamd_permute_quant_1x128_dual_grouped(const void* x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
                                                      const int64_t* sorted_idx, int topk, int64_t M,
                                                      const int64_t* group_offsets, int E, int32_t* tile_ws, uint8_t* q,
-                                                     float* s, uint8_t* q_t, float* s_t, int64_t ld_t, float eps,
-                                                     void* stream) {
+                                                     float* s, uint8_t* q_t, float* s_t, int64_t ld_t, int q_t_layout,
+                                                     float eps, void* stream) {
   AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "permute_quant_dual: unsupported dtype %d", x_dtype);
+  AAMD_REQUIRE(q_t_layout == AAMD_QT_ROWS || q_t_layout == AAMD_QT_BLOCKED, "permute_quant_dual: unknown q_t layout %d", q_t_layout);
   AAMD_REQUIRE(T >= 0 && M >= 0 && cols >= 0 && cols % kTile == 0, "permute_quant_dual: cols=%lld must be a multiple of 128",
                (long long)cols);
   AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "permute_quant_dual: bad ldx=%lld", (long long)ldx);
@@ -904,11 +920,11 @@ extern "C" int aamd_permute_quant_1x128_dual_grouped(const void* x, int x_dtype,
   dim3 grid((unsigned)(cols / kTile), (unsigned)grid_tiles), block(256);
   const int nt = (int)(cols / kTile);
   if (x_dtype == AAMD_BF16)
-    quant_dual_gather_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+    quant_dual_gather_kernel<BF16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, q_t_layout, eps);
   else if (x_dtype == AAMD_F16)
-    quant_dual_gather_kernel<F16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+    quant_dual_gather_kernel<F16><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, q_t_layout, eps);
   else
-    quant_dual_gather_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, eps);
+    quant_dual_gather_kernel<F32><<<grid, block, 0, st>>>((const float*)x, ldx, nt, sorted_idx, magic, sh, (uint32_t)T, group_offsets, tile_ws, E, q, s, q_t, s_t, ld_t, q_t_layout, eps);
   AAMD_LAUNCH_CHECK("permute_quant_dual_grouped");
   return AAMD_OK;
 }
@@ -938,7 +954,8 @@ extern "C" int aamd_swiglu_quant_1x128(const void* fc1, int64_t rows, int64_t F,
 extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, int64_t F, int64_t ld,
                                                     const int64_t* group_offsets, int E, int32_t* tile_ws,
                                                     void* h_out, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
-                                                    int64_t ld_t, void* stream) {
+                                                    int64_t ld_t, int q_t_layout, void* stream) {
+  AAMD_REQUIRE(q_t_layout == AAMD_QT_ROWS || q_t_layout == AAMD_QT_BLOCKED, "swiglu_quant_dual: unknown q_t layout %d", q_t_layout);
   AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "swiglu_quant_dual: F=%lld must be a multiple of 128", (long long)F);
   AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld < kMaxTileLd && ld_t < kMaxTileLd, "swiglu_quant_dual: bad ld=%lld", (long long)ld);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "swiglu_quant_dual: group_offsets / tile_ws required");
@@ -957,7 +974,7 @@ extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, 
   if (rc) return rc;
   dim3 grid((unsigned)(F / kTile), (unsigned)grid_tiles), block(256);
   quant_dual_grouped_kernel<GLU><<<grid, block, 0, st>>>((const u16*)fc1, ld, (int)(F / kTile), group_offsets, tile_ws, E,
-                                                         q, s, q_t, s_t, ld_t, 0.f, F, (u16*)h_out);
+                                                         q, s, q_t, s_t, ld_t, q_t_layout, 0.f, F, (u16*)h_out);
   AAMD_LAUNCH_CHECK("swiglu_quant_dual_grouped");
   return AAMD_OK;
 }
@@ -986,7 +1003,8 @@ extern "C" int aamd_gelu_quant_1x128(const void* x, int64_t rows, int64_t F, int
 extern "C" int aamd_gelu_quant_1x128_dual_grouped(const void* x, const void* dh, int64_t M, int64_t F, int64_t ld,
                                                   const int64_t* group_offsets, int E, int32_t* tile_ws, void* h_out,
                                                   uint8_t* q, float* s, uint8_t* q_t, float* s_t, int64_t ld_t,
-                                                  void* stream) {
+                                                  int q_t_layout, void* stream) {
+  AAMD_REQUIRE(q_t_layout == AAMD_QT_ROWS || q_t_layout == AAMD_QT_BLOCKED, "gelu_quant_dual: unknown q_t layout %d", q_t_layout);
   AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "gelu_quant_dual: F=%lld must be a multiple of 128", (long long)F);
   AAMD_REQUIRE(ld >= F && ld % 8 == 0 && ld < kMaxTileLd && ld_t < kMaxTileLd, "gelu_quant_dual: bad ld=%lld", (long long)ld);
   AAMD_REQUIRE(E >= 1 && group_offsets && tile_ws, "gelu_quant_dual: group_offsets / tile_ws required");
@@ -1007,11 +1025,11 @@ extern "C" int aamd_gelu_quant_1x128_dual_grouped(const void* x, const void* dh,
   dim3 grid((unsigned)(F / kTile), (unsigned)grid_tiles), block(256);
   if (dh == nullptr) {
     quant_dual_grouped_kernel<GELU><<<grid, block, 0, st>>>((const u16*)x, ld, (int)(F / kTile), group_offsets, tile_ws, E, q, s,
-                                                            q_t, s_t, ld_t, 0.f, 0, (u16*)h_out);
+                                                            q_t, s_t, ld_t, q_t_layout, 0.f, 0, (u16*)h_out);
   } else {
     const int64_t dh_off = (const u16*)dh - (const u16*)x;  // elements; the loader reads dh at x + dh_off
     quant_dual_grouped_kernel<GELUB><<<grid, block, 0, st>>>((const u16*)x, ld, (int)(F / kTile), group_offsets, tile_ws, E, q, s,
-                                                             q_t, s_t, ld_t, 0.f, dh_off, (u16*)h_out);
+                                                             q_t, s_t, ld_t, q_t_layout, 0.f, dh_off, (u16*)h_out);
   }
   AAMD_LAUNCH_CHECK("gelu_quant_dual_grouped");
   return AAMD_OK;
@@ -1020,7 +1038,9 @@ extern "C" int aamd_gelu_quant_1x128_dual_grouped(const void* x, const void* dh,
 extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t ld_dh, const void* fc1, int64_t ld,
                                                         int64_t M, int64_t F, const int64_t* group_offsets, int E,
                                                         int32_t* tile_ws, void* g_out, uint8_t* q, float* s,
-                                                        uint8_t* q_t, float* s_t, int64_t ld_t, void* stream) {
+                                                        uint8_t* q_t, float* s_t, int64_t ld_t, int q_t_layout,
+                                                        void* stream) {
+  AAMD_REQUIRE(q_t_layout == AAMD_QT_ROWS || q_t_layout == AAMD_QT_BLOCKED, "swiglu_bwd_quant_dual: unknown q_t layout %d", q_t_layout);
   AAMD_REQUIRE(M >= 0 && F >= 0 && F % kTile == 0, "swiglu_bwd_quant_dual: F=%lld must be a multiple of 128", (long long)F);
   AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld_dh >= F && ld_dh % 8 == 0 && ld < kMaxTileLd && ld_dh < kMaxTileLd && ld_t < kMaxTileLd,
                "swiglu_bwd_quant_dual: bad ld=%lld / ld_dh=%lld",
@@ -1043,7 +1063,7 @@ extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t 
   const int nt = (int)(2 * F / kTile);
   dim3 grid((unsigned)(nt / 2), (unsigned)grid_tiles), block(512);  // two teams: the da and the db tile of a feature tile
   swiglu_bwd_dual_kernel<<<grid, block, 0, st>>>((const u16*)fc1, ld, F, (const u16*)dh, ld_dh, nt, group_offsets, tile_ws, E,
-                                                 q, s, q_t, s_t, ld_t, (u16*)g_out);
+                                                 q, s, q_t, s_t, ld_t, q_t_layout, (u16*)g_out);
   AAMD_LAUNCH_CHECK("swiglu_bwd_quant_dual_grouped");
   return AAMD_OK;
 }

@@ -85,19 +85,19 @@ class _Fp8ExpertMlp(torch.autograd.Function):
             M = dispatch.sorted_indices.numel()
             if train:
                 qx, sx, qx_t, sx_t = kernels.permute_tile_quant_dual_grouped(
-                    xc, dispatch.sorted_indices, dispatch.topk, goff, E
+                    xc, dispatch.sorted_indices, dispatch.topk, goff, E, blocked=True
                 )
             else:  # every token quantised once, its codes written to its top-k rows
                 qx, sx = kernels.permute_tile_quant(xc, dispatch.row_map, dispatch.topk, M)
         elif train:
-            qx, sx, qx_t, sx_t = kernels.tile_quant_dual_grouped(xc, goff, E)
+            qx, sx, qx_t, sx_t = kernels.tile_quant_dual_grouped(xc, goff, E, blocked=True)
         else:
             qx, sx = kernels.tile_quant(xc)
         fc1 = kernels.grouped_gemm_nt(qx, sx, q1, s1, goff, out_dtype=torch.bfloat16,
                                       bias=b1.detach().contiguous() if b1 is not None else None)  # fmt: skip
         if train:
             quant = kernels.swiglu_tile_quant_dual_grouped if glu else kernels.gelu_tile_quant_dual_grouped
-            qh, sh, qh_t, sh_t = quant(fc1, goff, E)
+            qh, sh, qh_t, sh_t = quant(fc1, goff, E, ld_t=kernels.qt_ld(qx_t), blocked=True)
         else:
             qh, sh = kernels.swiglu_tile_quant(fc1) if glu else kernels.gelu_tile_quant(fc1)
         out = kernels.grouped_gemm_nt(qh, sh, q2_t, s2_t, goff, out_dtype=x.dtype,
@@ -119,20 +119,21 @@ class _Fp8ExpertMlp(torch.autograd.Function):
         x_dtype, w1_dtype, w2_dtype = ctx.dtypes
         dy = dy.contiguous().to(torch.bfloat16)
         M = dy.shape[0]
+        ld_t = kernels.qt_ld(qx_t)
         bin_ids = None
         if ctx.has_b1 or ctx.has_b2:  # expert of every row, from the device-side offsets (no host round trip)
             bin_ids = torch.repeat_interleave(torch.arange(E, device=dy.device), goff[1:] - goff[:-1], output_size=M)
         db2 = bias_gather_add_bw(dy, bin_ids, E) if ctx.has_b2 else None
-        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E)
+        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E, ld_t=ld_t, blocked=True)
         # through the second linear: dh = dy @ w2^T ([M, F]); dw2[f, h] = sum_m h[m, f] dy[m, h]
         dh = kernels.grouped_gemm_nt(qdy, sdy, q2, s2, goff, out_dtype=torch.bfloat16)
         dw2 = kernels.grouped_gemm_wgrad(qh_t, sh_t, qdy_t, sdy_t, goff, out_dtype=w2_dtype)
         # through the activation: the gradient of fc1 is quantised by the kernel that computes it and is
         # written in bf16 only when a bias gradient needs its row sums
         if ctx.glu:
-            res = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E, return_grad=ctx.has_b1)
+            res = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E, ld_t=ld_t, blocked=True, return_grad=ctx.has_b1)
         else:
-            res = kernels.gelu_tile_quant_dual_grouped(fc1, goff, E, dh=dh, return_activation=ctx.has_b1)
+            res = kernels.gelu_tile_quant_dual_grouped(fc1, goff, E, dh=dh, ld_t=ld_t, blocked=True, return_activation=ctx.has_b1)
         qg, sg, qg_t, sg_t = res[:4]
         db1 = bias_gather_add_bw(res[4], bin_ids, E) if ctx.has_b1 else None
         # through the first linear: dx = dfc1 @ w1 ([M, H]); dw1[n, h] = sum_m dfc1[m, n] x[m, h]

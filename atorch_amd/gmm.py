@@ -48,7 +48,7 @@ class _Fp8Gmm(torch.autograd.Function):
             w_q, w_s, wt_q, wt_s = qb_t, sb_t, qb, sb
         a_c = a.detach().contiguous()
         if need_grad:
-            qa, sa, qa_t, sa_t = kernels.tile_quant_dual_grouped(a_c, goff, E)
+            qa, sa, qa_t, sa_t = kernels.tile_quant_dual_grouped(a_c, goff, E, blocked=True)
         else:
             qa, sa = kernels.tile_quant(a_c)
             qa_t = sa_t = None
@@ -64,7 +64,7 @@ class _Fp8Gmm(torch.autograd.Function):
         goff, wt_q, wt_s, qa_t, sa_t = ctx.saved_tensors
         E = goff.numel() - 1
         dy = dy.contiguous()
-        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E)
+        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E, ld_t=kernels.qt_ld(qa_t), blocked=True)
         da = kernels.grouped_gemm_nt(qdy, sdy, wt_q, wt_s, goff, out_dtype=dy.dtype)
         # dW[g] = dY_g^T A_g -> [E, N, K]; for trans_b == False the parameter is [E, K, N]
         if ctx.trans_b:

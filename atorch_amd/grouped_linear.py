@@ -326,7 +326,7 @@ class _GroupedLinearDeviceOffsets(torch.autograd.Function):
         qw, sw, qw_t, sw_t = cached
 
         if is_grad_enabled:
-            qx, sx, qx_t, sx_t = kernels.tile_quant_dual_grouped(x2d, group_offsets, E, eps=qp.x_params.eps)
+            qx, sx, qx_t, sx_t = kernels.tile_quant_dual_grouped(x2d, group_offsets, E, eps=qp.x_params.eps, blocked=True)
         else:
             qx, sx = kernels.tile_quant(x2d, eps=qp.x_params.eps)
         bias = None
@@ -363,7 +363,9 @@ class _GroupedLinearDeviceOffsets(torch.autograd.Function):
             bin_ids = torch.repeat_interleave(torch.arange(E, device=dy.device), counts, output_size=M)
             g = dy2d if dy2d.dtype != torch.float16 else dy2d.float()
             bgrads = list(bias_gather_add_bw(g, bin_ids, E).to(dy.dtype).unbind(0))
-        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(dy2d, goff, E, eps=qp.g_params.eps, ld_t=qx_t.shape[1])
+        qdy, sdy, qdy_t, sdy_t = kernels.tile_quant_dual_grouped(
+            dy2d, goff, E, eps=qp.g_params.eps, ld_t=kernels.qt_ld(qx_t), blocked=True
+        )
         dgrad = kernels.grouped_gemm_nt(qdy, sdy, qw_t, sw_t, goff, out_dtype=f32_if_half(dgrad_dtype)).to(dgrad_dtype)
 
         if ctx.is_first_microbatch is not None:

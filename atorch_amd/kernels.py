@@ -166,6 +166,23 @@ def permute_rows(x: torch.Tensor, row_map: torch.Tensor, topk: int, num_out_rows
     return out
 
 
+def _alloc_qt(rows: int, ld_t: int, blocked: bool, dev) -> torch.Tensor:
+    """The transposed codes of ``rows`` columns and ``ld_t`` padded tokens: ``[rows, ld_t]``, or, blocked,
+    ``[ld_t/128, rows, 128]`` (token-block-major: every 128 x 128 tile is 16 KB of consecutive bytes)."""
+    shape = (ld_t // TILE, rows, TILE) if blocked else (rows, ld_t)
+    return torch.empty(shape, dtype=FP8, device=dev)
+
+
+def qt_ld(q_t: torch.Tensor) -> int:
+    """Padded token count ``ld_t`` of transposed codes in either layout."""
+    return q_t.shape[0] * TILE if q_t.dim() == 3 else q_t.shape[1]
+
+
+def qt_rows(q_t: torch.Tensor) -> torch.Tensor:
+    """Transposed codes of either layout as ``[rows, ld_t]`` (a copy for the blocked layout)."""
+    return q_t.permute(1, 0, 2).reshape(q_t.shape[1], -1) if q_t.dim() == 3 else q_t
+
+
 def tile_quant_dual_grouped(
     x: torch.Tensor,
     group_offsets: torch.Tensor,
@@ -173,13 +190,16 @@ def tile_quant_dual_grouped(
     eps: float = 0.0,
     ld_t: Optional[int] = None,
     rowwise: bool = True,
+    blocked: bool = False,
 ):
     """Row-wise and transposed 1x128 quantisation of ragged row groups in one pass.
 
     Returns ``(q [M,K], s [M,K/128], q_t [K, ld_t], s_t [ld_t/128, K])``; group g's transposed
     codes start at column ``sum_{j<g} ceil(M_j/128)*128`` and its partial last tile is zero
     padded.  ``ld_t`` defaults to a bound that needs no host knowledge of the splits.
-    With ``rowwise=False`` q and s are None.
+    With ``rowwise=False`` q and s are None.  With ``blocked=True`` q_t is ``[ld_t/128, K, 128]`` (the layout
+    the training path uses: the quantiser writes, and the weight-gradient GEMM reads, whole 16 KB tiles);
+    ``grouped_gemm_wgrad`` takes either.
     """
     assert x.dim() == 2 and x.is_contiguous()
     M, cols = x.shape
@@ -190,13 +210,13 @@ def tile_quant_dual_grouped(
     dev = x.device
     q = torch.empty((M, cols), dtype=FP8, device=dev) if rowwise else None
     s = torch.empty((M, cols // TILE), dtype=torch.float32, device=dev) if rowwise else None
-    q_t = torch.empty((cols, ld_t), dtype=FP8, device=dev)
+    q_t = _alloc_qt(cols, ld_t, blocked, dev)
     s_t = torch.empty((ld_t // TILE, cols), dtype=torch.float32, device=dev)
     ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
     check(
         lib().aamd_quant_1x128_dual_grouped(
             ptr(x), dtype_code(x.dtype, True), M, cols, cols, ptr(group_offsets), num_groups, ptr(ws),
-            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, eps, stream(),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, int(blocked), eps, stream(),
         )
     )  # fmt: skip
     return q, s, q_t, s_t
@@ -211,6 +231,7 @@ def permute_tile_quant_dual_grouped(
     eps: float = 0.0,
     ld_t: Optional[int] = None,
     rowwise: bool = True,
+    blocked: bool = False,
 ):
     """``tile_quant_dual_grouped`` of the permuted rows without materialising them: ``x [T, K]`` is in token
     order, permuted row j is token ``sorted_idx[j] // topk`` (``sorted_idx`` int64 ``[M]`` from
@@ -227,13 +248,13 @@ def permute_tile_quant_dual_grouped(
     dev = x.device
     q = torch.empty((M, cols), dtype=FP8, device=dev) if rowwise else None
     s = torch.empty((M, cols // TILE), dtype=torch.float32, device=dev) if rowwise else None
-    q_t = torch.empty((cols, ld_t), dtype=FP8, device=dev)
+    q_t = _alloc_qt(cols, ld_t, blocked, dev)
     s_t = torch.empty((ld_t // TILE, cols), dtype=torch.float32, device=dev)
     ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
     check(
         lib().aamd_permute_quant_1x128_dual_grouped(
             ptr(x), dtype_code(x.dtype, True), T, cols, cols, ptr(sorted_idx), topk, M, ptr(group_offsets), num_groups,
-            ptr(ws), ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, eps, stream(),
+            ptr(ws), ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, int(blocked), eps, stream(),
         )
     )  # fmt: skip
     return q, s, q_t, s_t
@@ -262,6 +283,7 @@ def swiglu_tile_quant_dual_grouped(
     num_groups: int,
     ld_t: Optional[int] = None,
     rowwise: bool = True,
+    blocked: bool = False,
     return_activation: bool = False,
 ):
     """SwiGLU fused into ``tile_quant_dual_grouped``: row-wise and transposed 1x128 quantisation of
@@ -277,14 +299,14 @@ def swiglu_tile_quant_dual_grouped(
     dev = fc1.device
     q = torch.empty((M, F), dtype=FP8, device=dev) if rowwise else None
     s = torch.empty((M, F // TILE), dtype=torch.float32, device=dev) if rowwise else None
-    q_t = torch.empty((F, ld_t), dtype=FP8, device=dev)
+    q_t = _alloc_qt(F, ld_t, blocked, dev)
     s_t = torch.empty((ld_t // TILE, F), dtype=torch.float32, device=dev)
     h = torch.empty((M, F), dtype=torch.bfloat16, device=dev) if return_activation else None
     ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
     check(
         lib().aamd_swiglu_quant_1x128_dual_grouped(
             ptr(fc1), M, F, two_f, ptr(group_offsets), num_groups, ptr(ws), ptr(h),
-            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, stream(),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, int(blocked), stream(),
         )
     )  # fmt: skip
     return (q, s, q_t, s_t, h) if return_activation else (q, s, q_t, s_t)
@@ -297,6 +319,7 @@ def swiglu_bwd_tile_quant_dual_grouped(
     num_groups: int,
     ld_t: Optional[int] = None,
     rowwise: bool = True,
+    blocked: bool = False,
     return_grad: bool = False,
 ):
     """Backward of ``h = silu(a) * b`` (rows ``[a | b]`` of ``fc1 [M, 2F]``) for the gradient
@@ -316,14 +339,14 @@ def swiglu_bwd_tile_quant_dual_grouped(
     dev = fc1.device
     q = torch.empty((M, two_f), dtype=FP8, device=dev) if rowwise else None
     s = torch.empty((M, two_f // TILE), dtype=torch.float32, device=dev) if rowwise else None
-    q_t = torch.empty((two_f, ld_t), dtype=FP8, device=dev)
+    q_t = _alloc_qt(two_f, ld_t, blocked, dev)
     s_t = torch.empty((ld_t // TILE, two_f), dtype=torch.float32, device=dev)
     g = torch.empty((M, two_f), dtype=torch.bfloat16, device=dev) if return_grad else None
     ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
     check(
         lib().aamd_swiglu_bwd_quant_1x128_dual_grouped(
             ptr(dh), F, ptr(fc1), two_f, M, F, ptr(group_offsets), num_groups, ptr(ws), ptr(g),
-            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, stream(),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, int(blocked), stream(),
         )
     )  # fmt: skip
     return (q, s, q_t, s_t, g) if return_grad else (q, s, q_t, s_t)
@@ -352,6 +375,7 @@ def gelu_tile_quant_dual_grouped(
     dh: Optional[torch.Tensor] = None,
     ld_t: Optional[int] = None,
     rowwise: bool = True,
+    blocked: bool = False,
     return_activation: bool = False,
 ):
     """GELU fused into ``tile_quant_dual_grouped``: quantises ``h = gelu(x)`` for ``x [M, F]`` bf16, or,
@@ -368,14 +392,14 @@ def gelu_tile_quant_dual_grouped(
     dev = x.device
     q = torch.empty((M, F), dtype=FP8, device=dev) if rowwise else None
     s = torch.empty((M, F // TILE), dtype=torch.float32, device=dev) if rowwise else None
-    q_t = torch.empty((F, ld_t), dtype=FP8, device=dev)
+    q_t = _alloc_qt(F, ld_t, blocked, dev)
     s_t = torch.empty((ld_t // TILE, F), dtype=torch.float32, device=dev)
     h = torch.empty((M, F), dtype=torch.bfloat16, device=dev) if return_activation else None
     ws = torch.empty(num_groups + 1, dtype=torch.int32, device=dev)
     check(
         lib().aamd_gelu_quant_1x128_dual_grouped(
             ptr(x), ptr(dh), M, F, F, ptr(group_offsets), num_groups, ptr(ws), ptr(h),
-            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, stream(),
+            ptr(q), ptr(s), ptr(q_t), ptr(s_t), ld_t, int(blocked), stream(),
         )
     )  # fmt: skip
     return (q, s, q_t, s_t, h) if return_activation else (q, s, q_t, s_t)
@@ -447,11 +471,14 @@ def grouped_gemm_wgrad(
     accumulate: bool = False,
 ) -> torch.Tensor:
     """dW[g] (+)= dY_g^T X_g from the transposed 1x128-quantised operands of
-    ``tile_quant_dual_grouped``: dy_t [N, ld_t], sdy_t [ld_t/128, N], x_t [K, ld_t], sx_t [ld_t/128, K]."""
-    N, ld_t = dy_t.shape
-    K = x_t.shape[0]
+    ``tile_quant_dual_grouped``: dy_t [N, ld_t], sdy_t [ld_t/128, N], x_t [K, ld_t], sx_t [ld_t/128, K], or
+    both code operands blocked, dy_t [ld_t/128, N, 128] and x_t [ld_t/128, K, 128]."""
+    blocked = dy_t.dim() == 3
+    assert x_t.dim() == dy_t.dim(), "both operands must be in the same layout"
+    N, K = (dy_t.shape[1], x_t.shape[1]) if blocked else (dy_t.shape[0], x_t.shape[0])
+    ld_t = qt_ld(dy_t)
     E = group_offsets.numel() - 1
-    assert x_t.shape[1] == ld_t and dy_t.is_contiguous() and x_t.is_contiguous()
+    assert qt_ld(x_t) == ld_t and dy_t.is_contiguous() and x_t.is_contiguous()
     assert sdy_t.shape == (ld_t // TILE, N) and sx_t.shape == (ld_t // TILE, K)
     assert sdy_t.is_contiguous() and sx_t.is_contiguous()
     if out is None:
@@ -460,7 +487,7 @@ def grouped_gemm_wgrad(
     assert out.shape == (E, N, K) and out.stride(2) == 1 and out.stride(1) == K
     ws = torch.empty(E + 1, dtype=torch.int32, device=dy_t.device)
     estride = out.stride(0) if E > 1 else N * K
-    args = (ptr(dy_t), ptr(sdy_t), ptr(x_t), ptr(sx_t), ld_t, ptr(group_offsets), E, ptr(ws), N, K,
+    args = (ptr(dy_t), ptr(sdy_t), ptr(x_t), ptr(sx_t), ld_t, int(blocked), ptr(group_offsets), E, ptr(ws), N, K,
             ptr(out), dtype_code(out.dtype), estride, int(accumulate))  # fmt: skip
     pinned = _pinned_options()
     if pinned:

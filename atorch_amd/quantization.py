@@ -453,7 +453,7 @@ class HipQuantizeOp:
             ws = torch.empty(E + 1, dtype=torch.int32, device=dev)
             check(
                 lib().aamd_grouped_gemm_fp8_wgrad(
-                    la[0], la[2], lb[0], lb[2], la[1], goff.data_ptr(), E, ws.data_ptr(), N, K,
+                    la[0], la[2], lb[0], lb[2], la[1], _lib.QT_ROWS, goff.data_ptr(), E, ws.data_ptr(), N, K,
                     oc[0], out_dt, oc[1], int(accumulate), stream(),
                 )
             )  # fmt: skip
@@ -476,7 +476,7 @@ class HipQuantizeOp:
             sxt = sx_t_list[e].t().contiguous()
             check(
                 lib().aamd_grouped_gemm_fp8_wgrad(
-                    dyt.data_ptr(), sdyt.data_ptr(), xt.data_ptr(), sxt.data_ptr(), ld, pairs[e].data_ptr(), 1,
+                    dyt.data_ptr(), sdyt.data_ptr(), xt.data_ptr(), sxt.data_ptr(), ld, _lib.QT_ROWS, pairs[e].data_ptr(), 1,
                     ws.data_ptr(), N, K, o.data_ptr(), out_dt, N * K, int(accumulate), stream(),
                 )
             )  # fmt: skip

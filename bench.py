@@ -368,9 +368,9 @@ class Layer:
         self.M, self.K, self.N, self.E = M, K, N, E
         self.goff = goff
         if backward:
-            self.qx, self.sx, self.qx_t, self.sx_t = kernels.tile_quant_dual_grouped(x, goff, E)
+            self.qx, self.sx, self.qx_t, self.sx_t = kernels.tile_quant_dual_grouped(x, goff, E, blocked=True)
             dy = randn((M, N), dev, 1e-2, seed + 2)
-            self.qdy, self.sdy, self.qdy_t, self.sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E)
+            self.qdy, self.sdy, self.qdy_t, self.sdy_t = kernels.tile_quant_dual_grouped(dy, goff, E, blocked=True)
             del dy
             self.qw, self.sw, self.qw_t, self.sw_t = kernels.block_quant_batched(w, return_transpose=True)
             self.dx = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
@@ -686,8 +686,8 @@ def run_c5(args, kernels, dev, cpu_baseline=True, mixes_too=None):
     t_sep, t_fused = Timer(), Timer()
     for i in range(2 + 5):
         for timer, fn in (
-            (t_sep, lambda: kernels.tile_quant_dual_grouped(kernels.permute_rows(x, row_map, k, M), goff, E)),
-            (t_fused, lambda: kernels.permute_tile_quant_dual_grouped(x, sorted_idx, k, goff, E)),
+            (t_sep, lambda: kernels.tile_quant_dual_grouped(kernels.permute_rows(x, row_map, k, M), goff, E, blocked=True)),
+            (t_fused, lambda: kernels.permute_tile_quant_dual_grouped(x, sorted_idx, k, goff, E, blocked=True)),
         ):
             a, b = timer.region() if i >= 2 else (None, None)
             if a is not None:
@@ -786,15 +786,15 @@ def run_quant(args, kernels, dev, steps=None, with_probe=True):
     # name: (call, algorithmic bytes, read:write mix of the streaming probe in equal-sized streams)
     cases = {
         "quant_1x128": (lambda: kernels.tile_quant(x), M * F * (2 + q1), "2:1"),
-        "quant_1x128_dual_grouped": (lambda: kernels.tile_quant_dual_grouped(x, goff, E), M * F * (2 + 2 * q1), "1:1"),
+        "quant_1x128_dual_grouped": (lambda: kernels.tile_quant_dual_grouped(x, goff, E, blocked=True), M * F * (2 + 2 * q1), "1:1"),
         "swiglu_quant_1x128": (lambda: kernels.swiglu_tile_quant(fc1), M * F * (4 + q1), "4:1"),
-        "swiglu_quant_1x128_dual_grouped": (lambda: kernels.swiglu_tile_quant_dual_grouped(fc1, goff, E),
+        "swiglu_quant_1x128_dual_grouped": (lambda: kernels.swiglu_tile_quant_dual_grouped(fc1, goff, E, blocked=True),
                                             M * F * (4 + 2 * q1), "2:1"),
-        "swiglu_bwd_quant_1x128_dual_grouped": (lambda: kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E),
+        "swiglu_bwd_quant_1x128_dual_grouped": (lambda: kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E, blocked=True),
                                                 M * F * (6 + 4 * q1), "3:2"),
-        "gelu_quant_1x128_dual_grouped": (lambda: kernels.gelu_tile_quant_dual_grouped(x, goff, E),
+        "gelu_quant_1x128_dual_grouped": (lambda: kernels.gelu_tile_quant_dual_grouped(x, goff, E, blocked=True),
                                           M * F * (2 + 2 * q1), "1:1"),
-        "gelu_bwd_quant_1x128_dual_grouped": (lambda: kernels.gelu_tile_quant_dual_grouped(x, goff, E, dh=dh),
+        "gelu_bwd_quant_1x128_dual_grouped": (lambda: kernels.gelu_tile_quant_dual_grouped(x, goff, E, dh=dh, blocked=True),
                                               M * F * (4 + 2 * q1), "2:1"),
         "quant_128x128": (lambda: kernels.block_quant_batched(w), w.numel() * 3, "2:1"),
         "quant_128x128_with_transpose": (lambda: kernels.block_quant_batched(w, return_transpose=True),

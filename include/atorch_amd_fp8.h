@@ -38,7 +38,16 @@ extern "C" {
 #define AAMD_F32 1
 #define AAMD_F16 2 /* accepted as the input type of the quantisers only */
 
-#define AAMD_ABI_VERSION 3
+/* Layouts of the transposed 1x128 codes q_t of R rows (columns of the quantised tensor) and ld_t padded tokens:
+ *   AAMD_QT_ROWS     q_t [R, ld_t]: one row of ld_t bytes per column of x;
+ *   AAMD_QT_BLOCKED  q_t [ld_t / 128, R, 128]: token-block-major, byte (r, t) at ((t / 128) * R + r) * 128 + t % 128.
+ * The second is what the grouped kernels use among themselves: a 128 x 128 tile of codes is 16 KB of consecutive
+ * bytes, which the quantisers write as one sequential sweep and the weight-gradient GEMM loads as whole slabs.
+ * The scales s_t [ld_t / 128, R] are the same in both. */
+#define AAMD_QT_ROWS 0
+#define AAMD_QT_BLOCKED 1
+
+#define AAMD_ABI_VERSION 4
 
 /* Library identity and error text. */
 int aamd_abi_version(void);
@@ -85,15 +94,15 @@ int aamd_permute_rows(const void *x, int x_dtype, int64_t T, int64_t cols, const
  * with a partial last token tile zero padded.
  *   x [M, cols]; group_offsets [E+1] int64 (device) exclusive prefix of rows per group;
  *   q [M, cols], s [M, cols/128]              (both may be NULL: transposed only)
- *   q_t [cols, ld_t]: q_t[c, poff_g + m] = code of x[off_g + m, c], where
- *       poff_g = sum_{j<g} ceil(M_j/128)*128; pad columns of a group are written 0
+ *   q_t, in the layout q_t_layout names: token poff_g + m of column c holds the code of x[off_g + m, c], where
+ *       poff_g = sum_{j<g} ceil(M_j/128)*128; pad tokens of a group are written 0
  *   s_t [ld_t/128, cols]: s_t[poff_g/128 + m/128, c]
  *   ld_t % 128 == 0 and ld_t >= poff_E (M + 127*E rounded up to 128 always suffices)
  *   tile_ws: E+1 int32 of scratch.
  */
 int aamd_quant_1x128_dual_grouped(const void *x, int x_dtype, int64_t M, int64_t cols, int64_t ldx,
                                   const int64_t *group_offsets, int E, int32_t *tile_ws, uint8_t *q, float *s,
-                                  uint8_t *q_t, float *s_t, int64_t ld_t, float eps, void *stream);
+                                  uint8_t *q_t, float *s_t, int64_t ld_t, int q_t_layout, float eps, void *stream);
 
 /*
  * The token permute fused into aamd_quant_1x128_dual_grouped: x holds the tokens in their original order and
@@ -105,14 +114,15 @@ int aamd_quant_1x128_dual_grouped(const void *x, int x_dtype, int64_t M, int64_t
  *   x [T, cols] (row stride ldx elements); sorted_idx [M] int64 (device): flat index token*topk+slot of
  *   permuted row j, the sorted_idx of aamd_moe_preprocess (M < T*topk when copies were dropped);
  *   T*topk < 2^31; group_offsets [E+1] int64 exclusive prefix of permuted rows per group;
- *   q [M, cols], s [M, cols/128] (both may be NULL), q_t [cols, ld_t], s_t [ld_t/128, cols], tile_ws and ld_t
+ *   q [M, cols], s [M, cols/128] (both may be NULL), q_t, s_t [ld_t/128, cols], tile_ws, ld_t and q_t_layout
  *   as for aamd_quant_1x128_dual_grouped.  Results equal aamd_permute_rows followed by
  *   aamd_quant_1x128_dual_grouped bit for bit.
  */
 int aamd_permute_quant_1x128_dual_grouped(const void *x, int x_dtype, int64_t T, int64_t cols, int64_t ldx,
                                           const int64_t *sorted_idx, int topk, int64_t M,
                                           const int64_t *group_offsets, int E, int32_t *tile_ws, uint8_t *q, float *s,
-                                          uint8_t *q_t, float *s_t, int64_t ld_t, float eps, void *stream);
+                                          uint8_t *q_t, float *s_t, int64_t ld_t, int q_t_layout, float eps,
+                                          void *stream);
 
 /*
  * 128x128 block quantisation of E weight matrices, optionally also emitting the
@@ -151,7 +161,8 @@ int aamd_swiglu_quant_1x128(const void *fc1, int64_t rows, int64_t F, int64_t ld
                             void *stream);
 int aamd_swiglu_quant_1x128_dual_grouped(const void *fc1, int64_t M, int64_t F, int64_t ld,
                                          const int64_t *group_offsets, int E, int32_t *tile_ws, void *h_out,
-                                         uint8_t *q, float *s, uint8_t *q_t, float *s_t, int64_t ld_t, void *stream);
+                                         uint8_t *q, float *s, uint8_t *q_t, float *s_t, int64_t ld_t, int q_t_layout,
+                                         void *stream);
 
 /*
  * Backward of the gated activation fused into the quantisation of its gradient: for the gradient dh
@@ -162,13 +173,13 @@ int aamd_swiglu_quant_1x128_dual_grouped(const void *fc1, int64_t M, int64_t F, 
  * calls of the first grouped linear's backward, quantized_grouped_linear.py:202-206.
  *   dh [M, F] bf16 (row stride ld_dh), fc1 [M, 2F] bf16 (row stride ld), F % 128 == 0
  *   g_out [M, 2F] bf16 or NULL (the gradient itself, for callers that keep it)
- *   q [M, 2F], s [M, 2F/128] (both may be NULL), q_t [2F, ld_t], s_t [ld_t/128, 2F];
- *   group_offsets, tile_ws, ld_t as for aamd_quant_1x128_dual_grouped.
+ *   q [M, 2F], s [M, 2F/128] (both may be NULL), q_t (2F rows), s_t [ld_t/128, 2F];
+ *   group_offsets, tile_ws, ld_t, q_t_layout as for aamd_quant_1x128_dual_grouped.
  */
 int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void *dh, int64_t ld_dh, const void *fc1, int64_t ld, int64_t M,
                                              int64_t F, const int64_t *group_offsets, int E, int32_t *tile_ws,
                                              void *g_out, uint8_t *q, float *s, uint8_t *q_t, float *s_t,
-                                             int64_t ld_t, void *stream);
+                                             int64_t ld_t, int q_t_layout, void *stream);
 
 /*
  * GELU, the expert MLP's default activation, fused into the same quantisers:
@@ -185,7 +196,7 @@ int aamd_gelu_quant_1x128(const void *x, int64_t rows, int64_t F, int64_t ld, vo
                           void *stream);
 int aamd_gelu_quant_1x128_dual_grouped(const void *x, const void *dh, int64_t M, int64_t F, int64_t ld,
                                        const int64_t *group_offsets, int E, int32_t *tile_ws, void *h_out, uint8_t *q,
-                                       float *s, uint8_t *q_t, float *s_t, int64_t ld_t, void *stream);
+                                       float *s, uint8_t *q_t, float *s_t, int64_t ld_t, int q_t_layout, void *stream);
 
 /*
  * Ragged grouped block-scaled GEMM, "NT": for every group g and its rows m,
@@ -225,15 +236,17 @@ int aamd_grouped_gemm_fp8_nt_static(const uint8_t *a, int64_t lda, const float *
  * aamd_quant_1x128_dual_grouped's q_t / s_t).
  * Replaces quantize_op.grouped_qgemm(qdy_t, qx_t, mm_wgrad, ..., accumulate=...),
  * quantized_grouped_linear.py:243-253.
- *   dyt [N, ld_t], sdyt [ld_t/128, N]; xt [K, ld_t], sxt [ld_t/128, K]
+ *   dyt (N rows), sdyt [ld_t/128, N]; xt (K rows), sxt [ld_t/128, K]; both code operands in the layout
+ *   q_t_layout names (AAMD_QT_ROWS: [N, ld_t] and [K, ld_t]; AAMD_QT_BLOCKED: [ld_t/128, N, 128] and
+ *   [ld_t/128, K, 128])
  *   dw [E, N, K] of dw_dtype (expert stride in elements); an empty group gives zeros,
  *   or leaves dw_g untouched when accumulate != 0.
  *   ld_t must cover the padded token total sum_g ceil(M_g/128)*128, which only the device knows:
  *   a group whose tokens lie beyond ld_t gets NaN in its dw_g instead of a wrong finite gradient.
  */
 int aamd_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uint8_t *xt, const float *sxt,
-                                int64_t ld_t, const int64_t *group_offsets, int E, int32_t *tile_ws, int64_t N,
-                                int64_t K, void *dw, int dw_dtype, int64_t expert_stride, int accumulate,
+                                int64_t ld_t, int q_t_layout, const int64_t *group_offsets, int E, int32_t *tile_ws,
+                                int64_t N, int64_t K, void *dw, int dw_dtype, int64_t expert_stride, int accumulate,
                                 void *stream);
 
 /*

@@ -34,9 +34,9 @@ int aamd_tuning_grouped_gemm_fp8_nt(const uint8_t *a, int64_t lda, const float *
                                     int32_t *tile_ws, int64_t M, int64_t N, int64_t K, void *c, int c_dtype,
                                     int64_t ldc, const void *bias, int bias_dtype, const int *opts, void *stream);
 int aamd_tuning_grouped_gemm_fp8_wgrad(const uint8_t *dyt, const float *sdyt, const uint8_t *xt, const float *sxt,
-                                       int64_t ld_t, const int64_t *group_offsets, int E, int32_t *tile_ws, int64_t N,
-                                       int64_t K, void *dw, int dw_dtype, int64_t expert_stride, int accumulate,
-                                       const int *opts, void *stream);
+                                       int64_t ld_t, int q_t_layout, const int64_t *group_offsets, int E,
+                                       int32_t *tile_ws, int64_t N, int64_t K, void *dw, int dw_dtype,
+                                       int64_t expert_stride, int accumulate, const int *opts, void *stream);
 
 /*
  * Shader clock probe (no counterpart in the reference; the benchmark reports the clock the GEMMs

@@ -164,14 +164,18 @@ def test_permute_quant_dual_grouped_full_size(oracle, dev, T, E, k, H, heavy):
     """The training form of the fused permute at the sizes of the quant / permute configuration (65536 x 7168, top-8
     into 64 experts) and of the Qwen-like one: equal to permute_rows followed by the dual grouped quantiser bit for
     bit over the whole outputs, its row-wise part equal to the scatter form (every token quantised once), and sampled
-    columns of sampled groups against the oracle."""
+    columns of sampled groups against the oracle.  The fused kernel writes its transposed codes token-block-major,
+    the separate ones a row per column: the comparison covers both layouts."""
     from atorch_amd import kernels as K
 
     x = _student_t((T, H), dev, seed=0) if heavy else _randn((T, H), dev, 1.0, 7)
     idx, _ = _routing(T, E, k, dev)
     sorted_idx, row_map, goff = K.moe_preprocess(idx, E)
     M = T * k
-    q, s, q_t, s_t = K.permute_tile_quant_dual_grouped(x, sorted_idx, k, goff, E)
+    # the token-block-major layout the training path uses, compared below with the row layout of the separate kernels
+    q, s, q_tb, s_t = K.permute_tile_quant_dual_grouped(x, sorted_idx, k, goff, E, blocked=True)
+    q_t = K.qt_rows(q_tb)
+    del q_tb
     counts = (goff[1:] - goff[:-1]).cpu().tolist()
     pad = [0]
     for c in counts:
