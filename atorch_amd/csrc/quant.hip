@@ -200,11 +200,33 @@ __device__ __forceinline__ v4i pack8_bf16(const float* v) {
 // 1x128 quant, 16 lanes per tile, U tiles per lane group.  SCATTER: write each quantised
 // row to its topk destinations (row_map), reading it once.
 // ---------------------------------------------------------------------------------------
+// floor(n / d) for n < 2^31 as one widening multiply and a shift: magic = floor(2^sh / d) + 1, sh = 31 + ceil(log2 d)
+struct FastDiv {
+  uint32_t magic;
+  int sh;
+  __device__ __forceinline__ uint32_t div(uint32_t n) const { return (uint32_t)(((uint64_t)n * magic) >> sh); }
+};
+static FastDiv make_fastdiv(uint32_t d) {
+  int l = 0;
+  while (((uint64_t)1 << l) < d) l++;
+  FastDiv f;
+  f.sh = 31 + l;
+  f.magic = (uint32_t)((((uint64_t)1 << f.sh) / (uint64_t)d) + 1);
+  return f;
+}
+
 // tiles per 16-lane group and pass: two keep enough loads in flight (one and four measured slower)
 constexpr int kQuantU = 2;
+constexpr int64_t kMaxRowLd = (int64_t)1 << 24;  // row strides (elements) of the row-wise quantisers' inputs
+// A workgroup takes 16 U consecutive tiles of the row-major tile order.  These kernels run close to the rate at
+// which the vector ALUs issue, so nothing that is the same in every lane is computed in the lanes: the position
+// of the block's first tile comes from the scalar unit, a lane adds its small tile number to it, and every
+// access is a scalar base plus a 32-bit lane offset.  The outputs are dense, so tile t of the order lies at
+// byte 128 t of q; the input needs (row, column tile) only where its rows are strided.
+// (the launchers keep ldx below 2^24: 16 U rows of it stay within the 32-bit offset)
 template <typename IN, bool SCATTER, int U>
 __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::elem* __restrict__ x, int64_t ldx,
-                                                          int nt, int64_t total_tiles,
+                                                          int nt, FastDiv nt_div, int64_t total_tiles,
                                                           const int32_t* __restrict__ row_map, int topk,
                                                           int64_t M_out, uint8_t* __restrict__ q,
                                                           float* __restrict__ s, float eps, int64_t gate_off,
@@ -212,22 +234,44 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
   // the short division is checked for bf16 values over scales of bf16 maxima only
   const bool plain_div = !kBf16Values<IN> || eps != 0.f;
   const int grp = threadIdx.x >> 4, l = threadIdx.x & 15;
-  const int64_t base = (int64_t)blockIdx.x * (16 * U);
+  constexpr uint32_t kEl = sizeof(typename IN::elem);
+  const int64_t base = (int64_t)blockIdx.x * (16 * U);  // first tile of the block: the same in every lane
+  const int64_t tiles_left = total_tiles - base;
+  const uint32_t left = tiles_left < 16 * U ? (uint32_t)tiles_left : 16u * U;  // >= 1
   const int64_t cols = (int64_t)nt * kTile;
+  const bool dense = !SCATTER && ldx == cols;
+  int64_t row0 = 0;
+  uint32_t tc0 = 0;
+  if (!dense) {
+    row0 = total_tiles < ((int64_t)1 << 31) ? (int64_t)nt_div.div((uint32_t)base) : base / nt;
+    tc0 = (uint32_t)(base - row0 * nt);
+  }
+  const typename IN::elem* const xb = dense ? x + base * kTile : x + row0 * ldx;
 
   Raw8<IN> raw[U];
-  int64_t row[U];
-  int tc[U];
+  uint32_t jt[U], wrow[U], tc[U];
   bool valid[U];
 #pragma unroll
   for (int u = 0; u < U; u++) {
-    int64_t tile = base + u * 16 + grp;
-    valid[u] = tile < total_tiles;
-    if (!valid[u]) tile = total_tiles - 1;
-    row[u] = tile / nt;
-    tc[u] = (int)(tile - row[u] * nt);
-    raw[u].load(x + row[u] * ldx + (int64_t)tc[u] * kTile + l * 8, 0u, gate_off);
+    uint32_t j = (uint32_t)(u * 16 + grp);
+    valid[u] = j < left;
+    if (!valid[u]) j = left - 1;
+    jt[u] = j;
+    uint32_t xoff;  // elements from xb
+    if (dense) {
+      xoff = j * kTile;
+      wrow[u] = tc[u] = 0;
+    } else {
+      const uint32_t t = tc0 + j;  // below nt + 16 U
+      wrow[u] = nt >= 16 * U ? (t >= (uint32_t)nt ? 1u : 0u) : nt_div.div(t);
+      tc[u] = t - wrow[u] * (uint32_t)nt;
+      xoff = wrow[u] * (uint32_t)ldx + tc[u] * kTile;
+    }
+    raw[u].load(xb, (xoff + (uint32_t)l * 8) * kEl, gate_off);
   }
+  u16* const hb = h_out ? h_out + base * kTile : nullptr;
+  uint8_t* const qb = q + base * kTile;
+  float* const sb = s + base;
 #pragma unroll
   for (int u = 0; u < U; u++) {
     float v[8];
@@ -236,18 +280,18 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const typename IN::ele
     const float sc = dv.s;
     const v2i codes = quant8(v, dv);
     if (!valid[u]) continue;
-    if (h_out != nullptr)  // the gated activation itself, for callers that keep it
-      __builtin_nontemporal_store(pack8_bf16(v), reinterpret_cast<v4i*>(h_out + row[u] * cols + (int64_t)tc[u] * kTile + l * 8));
+    const uint32_t off = jt[u] * kTile + (uint32_t)l * 8;  // element of the dense outputs, from the block's first tile
+    if (h_out != nullptr) st_nt(hb, off * 2, pack8_bf16(v));  // the activation itself, for callers that keep it
     // the codes are not read again by this kernel: streaming stores keep them out of the way
-    auto put = [&](v2i* dst, v2i val) { __builtin_nontemporal_store(val, dst); };
     if constexpr (!SCATTER) {
-      put(reinterpret_cast<v2i*>(q + row[u] * cols + (int64_t)tc[u] * kTile + l * 8), codes);
-      if (l == 0) s[row[u] * nt + tc[u]] = sc;
+      st_nt(qb, off, codes);
+      if (l == 0) sb[jt[u]] = sc;
     } else {
+      const int64_t row = row0 + wrow[u];
       for (int j = 0; j < topk; j++) {
-        const int64_t dst = row_map[row[u] * topk + j];
+        const int64_t dst = row_map[row * topk + j];
         if (dst < 0 || dst >= M_out) continue;
-        put(reinterpret_cast<v2i*>(q + dst * cols + (int64_t)tc[u] * kTile + l * 8), codes);
+        __builtin_nontemporal_store(codes, reinterpret_cast<v2i*>(q + dst * cols + (int64_t)tc[u] * kTile + l * 8));
         if (l == 0) s[dst * nt + tc[u]] = sc;
       }
     }
@@ -814,7 +858,7 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   AAMD_REQUIRE(x_dtype == AAMD_BF16 || x_dtype == AAMD_F32 || x_dtype == AAMD_F16, "quant_1x128: unsupported dtype %d", x_dtype);
   AAMD_REQUIRE(T >= 0 && cols >= 0 && cols % kTile == 0, "quant_1x128: cols=%lld must be a multiple of 128",
                (long long)cols);
-  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0, "quant_1x128: ldx=%lld must be >= cols and a multiple of 8",
+  AAMD_REQUIRE(ldx >= cols && ldx % 8 == 0 && ldx < kMaxRowLd, "quant_1x128: ldx=%lld must be >= cols, a multiple of 8 and below 2^24",
                (long long)ldx);
   AAMD_REQUIRE(topk >= 1 && M_out >= 0, "quant_1x128: bad topk/M_out");
   if (T == 0 || cols == 0) return AAMD_OK;
@@ -828,20 +872,21 @@ extern "C" int aamd_permute_quant_1x128(const void* x, int x_dtype, int64_t T, i
   const int64_t blocks = (total + 16 * U - 1) / (16 * U);
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "quant_1x128: grid too large");
   dim3 grid((unsigned)blocks), block(256);
+  const FastDiv nd = make_fastdiv((uint32_t)nt);
   if (row_map == nullptr) {
     if (x_dtype == AAMD_BF16)
-      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
+      quant_1x128_kernel<BF16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, nd, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
     else if (x_dtype == AAMD_F16)
-      quant_1x128_kernel<F16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
+      quant_1x128_kernel<F16, false, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, nd, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
     else
-      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
+      quant_1x128_kernel<F32, false, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, nd, total, nullptr, 1, M_out, q, s, eps, 0, nullptr);
   } else {
     if (x_dtype == AAMD_BF16)
-      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
+      quant_1x128_kernel<BF16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, nd, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
     else if (x_dtype == AAMD_F16)
-      quant_1x128_kernel<F16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
+      quant_1x128_kernel<F16, true, U><<<grid, block, 0, st>>>((const u16*)x, ldx, nt, nd, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
     else
-      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
+      quant_1x128_kernel<F32, true, U><<<grid, block, 0, st>>>((const float*)x, ldx, nt, nd, total, row_map, topk, M_out, q, s, eps, 0, nullptr);
   }
   AAMD_LAUNCH_CHECK("quant_1x128");
   return AAMD_OK;
@@ -935,7 +980,7 @@ extern "C" int aamd_permute_quant_1x128_dual_grouped(const void* x, int x_dtype,
 extern "C" int aamd_swiglu_quant_1x128(const void* fc1, int64_t rows, int64_t F, int64_t ld, void* h_out, uint8_t* q,
                                        float* s, void* stream) {
   AAMD_REQUIRE(rows >= 0 && F >= 0 && F % kTile == 0, "swiglu_quant: F=%lld must be a multiple of 128", (long long)F);
-  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0, "swiglu_quant: ld=%lld must be >= 2F and a multiple of 8", (long long)ld);
+  AAMD_REQUIRE(ld >= 2 * F && ld % 8 == 0 && ld < kMaxRowLd, "swiglu_quant: ld=%lld must be >= 2F, a multiple of 8 and below 2^24", (long long)ld);
   if (rows == 0 || F == 0) return AAMD_OK;
   AAMD_REQUIRE(fc1 && q && s, "swiglu_quant: null pointer");
   AAMD_REQUIRE(aligned16(fc1) && aligned16(q) && aligned16(h_out), "swiglu_quant: pointers must be 16-byte aligned");
@@ -946,7 +991,7 @@ extern "C" int aamd_swiglu_quant_1x128(const void* fc1, int64_t rows, int64_t F,
   const int64_t blocks = (total + 16 * U - 1) / (16 * U);
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "swiglu_quant: grid too large");
   quant_1x128_kernel<GLU, false, U><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-      (const u16*)fc1, ld, nt, total, nullptr, 1, rows, q, s, 0.f, F, (u16*)h_out);
+      (const u16*)fc1, ld, nt, make_fastdiv((uint32_t)nt), total, nullptr, 1, rows, q, s, 0.f, F, (u16*)h_out);
   AAMD_LAUNCH_CHECK("swiglu_quant_1x128");
   return AAMD_OK;
 }
@@ -983,7 +1028,7 @@ extern "C" int aamd_swiglu_quant_1x128_dual_grouped(const void* fc1, int64_t M, 
 extern "C" int aamd_gelu_quant_1x128(const void* x, int64_t rows, int64_t F, int64_t ld, void* h_out, uint8_t* q, float* s,
                                      void* stream) {
   AAMD_REQUIRE(rows >= 0 && F >= 0 && F % kTile == 0, "gelu_quant: F=%lld must be a multiple of 128", (long long)F);
-  AAMD_REQUIRE(ld >= F && ld % 8 == 0, "gelu_quant: ld=%lld must be >= F and a multiple of 8", (long long)ld);
+  AAMD_REQUIRE(ld >= F && ld % 8 == 0 && ld < kMaxRowLd, "gelu_quant: ld=%lld must be >= F, a multiple of 8 and below 2^24", (long long)ld);
   if (rows == 0 || F == 0) return AAMD_OK;
   AAMD_REQUIRE(x && q && s, "gelu_quant: null pointer");
   AAMD_REQUIRE(aligned16(x) && aligned16(q) && aligned16(h_out), "gelu_quant: pointers must be 16-byte aligned");
@@ -994,7 +1039,7 @@ extern "C" int aamd_gelu_quant_1x128(const void* x, int64_t rows, int64_t F, int
   const int64_t blocks = (total + 16 * U - 1) / (16 * U);
   AAMD_REQUIRE(blocks < 0x7fffffffLL, "gelu_quant: grid too large");
   quant_1x128_kernel<GELU, false, U><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-      (const u16*)x, ld, nt, total, nullptr, 1, rows, q, s, 0.f, 0, (u16*)h_out);
+      (const u16*)x, ld, nt, make_fastdiv((uint32_t)nt), total, nullptr, 1, rows, q, s, 0.f, 0, (u16*)h_out);
   AAMD_LAUNCH_CHECK("gelu_quant_1x128");
   return AAMD_OK;
 }

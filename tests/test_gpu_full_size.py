@@ -282,6 +282,12 @@ def _check_wgrad(K_, ops, goff, E, N, Kd, dev, seed):
     dw2 = dw.clone()
     K_.grouped_gemm_wgrad(ops["qdy_t"], ops["sdy_t"], ops["qx_t"], ops["sx_t"], goff, out=dw2, accumulate=True)
     assert torch.equal(dw2, dw + dw)
+    del dw2
+    # the token-block-major operand layout [ld_t/128, rows, 128] (what the training path hands over), made here by
+    # plain torch from the row layout: the same bits
+    blk = lambda t: t.view(torch.uint8).view(t.shape[0], -1, TILE).permute(1, 0, 2).contiguous().view(FP8)  # noqa: E731
+    dwb = K_.grouped_gemm_wgrad(blk(ops["qdy_t"]), ops["sdy_t"], blk(ops["qx_t"]), ops["sx_t"], goff)
+    assert torch.equal(dwb, dw)
 
 
 def test_grouped_gemm_mixtral_full_size(dev):

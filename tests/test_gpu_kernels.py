@@ -179,6 +179,74 @@ def test_tile_quant_matches_oracle(oracle, dev, dtype, shape):
     assert torch.equal(_u8(q), qo)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,cols,pad", [(37, 128, 8), (50, 384, 64), (21, 5120, 128), (3, 4096 + 128, 1 << 20)])
+def test_tile_quant_of_strided_rows_and_scatter_through_the_c_abi(oracle, dev, dtype, rows, cols, pad):
+    """Rows ldx = cols + pad elements apart (a column slice of a wider tensor), which only the C entry point takes:
+    the same codes as the dense copy, for tile counts per row below and above a workgroup's 32 tiles and row counts
+    that leave the last workgroup partly filled; and the scatter form (every row to two destinations) on the same
+    strided input."""
+    import ctypes
+
+    from atorch_amd import _lib
+
+    L = _lib.lib()
+    wide = heavy_tailed((rows, cols + pad), seed=rows + cols, dtype=dtype).to(dev) if pad < 4096 else None
+    if wide is None:  # a stride of a million elements: only the rows themselves are allocated densely elsewhere
+        buf = torch.zeros(rows * (cols + pad), dtype=dtype, device=dev)
+        wide = buf.view(rows, cols + pad)
+        wide[:, :cols] = heavy_tailed((rows, cols), seed=rows + cols, dtype=dtype).to(dev)
+    x = wide[:, :cols]
+    qo, so = oracle.tile_quant(x.cpu().contiguous())
+    vp = ctypes.c_void_p
+    q = torch.zeros((rows, cols), dtype=torch.uint8, device=dev)
+    sc = torch.zeros((rows, cols // TILE), dtype=torch.float32, device=dev)
+    st = vp(torch.cuda.current_stream().cuda_stream)
+    code = _lib.dtype_code(dtype)
+    rc = L.aamd_quant_1x128(vp(x.data_ptr()), code, rows, cols, cols + pad, vp(q.data_ptr()), vp(sc.data_ptr()), 0.0, st)
+    assert rc == _lib.OK, L.aamd_last_error()
+    assert torch.equal(q.cpu(), qo) and torch.equal(sc.cpu(), so)
+    # scatter: row r goes to rows r and rows + (rows - 1 - r) of a [2 rows, cols] output
+    row_map = torch.stack([torch.arange(rows), 2 * rows - 1 - torch.arange(rows)], 1).to(torch.int32).to(dev).contiguous()
+    q2 = torch.zeros((2 * rows, cols), dtype=torch.uint8, device=dev)
+    s2 = torch.zeros((2 * rows, cols // TILE), dtype=torch.float32, device=dev)
+    rc = L.aamd_permute_quant_1x128(vp(x.data_ptr()), code, rows, cols, cols + pad, vp(row_map.data_ptr()), 2, 2 * rows,
+                                    vp(q2.data_ptr()), vp(s2.data_ptr()), 0.0, st)
+    assert rc == _lib.OK, L.aamd_last_error()
+    assert torch.equal(q2[:rows].cpu(), qo) and torch.equal(q2[rows:].flip(0).cpu(), qo)
+    assert torch.equal(s2[:rows].cpu(), so) and torch.equal(s2[rows:].flip(0).cpu(), so)
+    # a row stride of 2^24 elements or more is refused
+    rc = L.aamd_quant_1x128(vp(x.data_ptr()), code, 1, cols, 1 << 24, vp(q.data_ptr()), vp(sc.data_ptr()), 0.0, st)
+    assert rc == _lib.ERR_ARG and b"2^24" in L.aamd_last_error()
+
+
+def test_swiglu_quant_of_wide_and_strided_rows(oracle, dev):
+    """The gated width above a workgroup's 32 tiles (F = 4224: 33 tiles per row) and rows ld > 2F apart, through the
+    C entry point: codes and scales equal to the 1x128 quantisation of the kernel's own activation."""
+    import ctypes
+
+    from atorch_amd import _lib, kernels
+
+    L = _lib.lib()
+    rows, F, ld = 19, 4224, 2 * 4224 + 256
+    wide = randn_bf16((rows, ld), 41, std=2.0).to(dev)
+    q = torch.zeros((rows, F), dtype=torch.uint8, device=dev)
+    sc = torch.zeros((rows, F // TILE), dtype=torch.float32, device=dev)
+    h = torch.zeros((rows, F), dtype=torch.bfloat16, device=dev)
+    vp = ctypes.c_void_p
+    rc = L.aamd_swiglu_quant_1x128(vp(wide.data_ptr()), rows, F, ld, vp(h.data_ptr()), vp(q.data_ptr()), vp(sc.data_ptr()),
+                                   vp(torch.cuda.current_stream().cuda_stream))
+    assert rc == _lib.OK, L.aamd_last_error()
+    q1, s1, h1 = kernels.swiglu_tile_quant(wide[:, : 2 * F].contiguous(), return_activation=True)
+    assert torch.equal(h, h1) and torch.equal(q, _u8q(q1)) and torch.equal(sc, s1)
+    ho = oracle.swiglu(wide[:, : 2 * F].cpu().contiguous())
+    d = _ulp_diff(h.cpu(), ho)
+    d = torch.where(h.cpu().float() == ho.float(), torch.zeros_like(d), d)
+    assert int(d.max()) <= 2
+    qo, so = oracle.tile_quant(h.cpu())
+    assert torch.equal(q.cpu(), qo) and torch.equal(sc.cpu(), so)
+
+
 def test_tile_quant_all_bf16_patterns(oracle, dev):
     """Every bf16 bit pattern as an element, for several tile maxima: pins the division and the
     hardware fp8 conversion (RNE, subnormals) against the integer encoder of the oracle."""
