@@ -141,6 +141,55 @@ __device__ __forceinline__ float gelu_phi(float x, float* exp_neg_half_sq = null
   const float h = q * e;  // erfc(t) / 2
   return x < 0.f ? h : 1.0f - h;
 }
+// Both GELU forms are functions of one bf16 value, x Phi(x) rounded to bf16 and Phi(x) + x pdf(x) in fp32, and cost
+// two dozen vector instructions per value, which is what bounds the fused kernels.  The dual kernels therefore read
+// them from tables in LDS indexed by the bits of x, for |x| in [2^-14, 2^3) (17 binades x 128 x 2 signs); values
+// outside (exact zeros, outliers) take the arithmetic.  The tables are filled by the same functions, by a small
+// kernel ahead of every launch, into arrays of the library on the device: every call writes the same values, so
+// calls that overlap do not disturb each other.
+constexpr uint32_t kLutLo = (uint32_t)(127 - 14) << 7;        // first magnitude (bits without the sign) of the tables
+constexpr uint32_t kLutN = (uint32_t)(14 + 3) << 7;           // magnitudes per sign
+static __device__ __attribute__((aligned(16))) u16 g_gelu_lut[2 * kLutN];
+static __device__ __attribute__((aligned(16))) float g_gelub_lut[2 * kLutN];
+__device__ __forceinline__ float gelu_grad_factor(float x) {
+  float e;  // exp(-x^2 / 2)
+  const float cdf = gelu_phi(x, &e);
+  const float pdf = 0.39894228040143267794f * e;
+  return cdf + x * pdf;
+}
+__global__ __launch_bounds__(256) void gelu_lut_kernel() {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= 2 * kLutN) return;
+  const uint32_t sign = i >= kLutN ? 1u : 0u;
+  const float x = __uint_as_float(((sign << 15) | (kLutLo + i - sign * kLutN)) << 16);
+  g_gelu_lut[i] = (u16)f32_to_bf16_bits(x * gelu_phi(x));
+  g_gelub_lut[i] = gelu_grad_factor(x);
+}
+// a pair of values outside the tables: out of line, these are rare
+__device__ __attribute__((noinline)) uint32_t gelu_pair_plain(uint32_t w) {
+  const float x0 = __uint_as_float(w << 16), x1 = __uint_as_float(w & 0xffff0000u);
+  return pack_bf16x2(x0 * gelu_phi(x0), x1 * gelu_phi(x1));
+}
+__device__ __attribute__((noinline)) uint32_t gelu_grad_pair_plain(uint32_t w, uint32_t gw) {
+  const float x0 = __uint_as_float(w << 16), x1 = __uint_as_float(w & 0xffff0000u);
+  const float g0 = __uint_as_float(gw << 16), g1 = __uint_as_float(gw & 0xffff0000u);
+  return pack_bf16x2(g0 * gelu_grad_factor(x0), g1 * gelu_grad_factor(x1));
+}
+// Table position of the bf16 value whose magnitude bits are `mag` and whose sign is `sign` (0 / 1); `ok` is cleared
+// when the value lies outside the tables (position 0 is returned then, so the read that follows stays inside).
+__device__ __forceinline__ uint32_t lut_index(uint32_t mag, uint32_t sign, bool& ok) {
+  const uint32_t m = mag - kLutLo;
+  const bool in = m < kLutN;
+  ok = ok && in;
+  return in ? m + sign * kLutN : 0u;
+}
+template <typename IN>
+constexpr uint32_t kLutBytes = 0;
+template <>
+constexpr uint32_t kLutBytes<GELU> = 2 * kLutN * sizeof(u16);
+template <>
+constexpr uint32_t kLutBytes<GELUB> = 2 * kLutN * sizeof(float);
+
 template <>
 struct Raw8<GELU> {
   v4i a;
@@ -159,6 +208,33 @@ struct Raw8<GELU> {
       v[i + 1] = __uint_as_float(h & 0xffff0000u);
     }
   }
+  // the same values from the table (a copy of g_gelu_lut in LDS): all eight reads are issued together, and a
+  // value outside the table, which is rare, sends its pair through the arithmetic afterwards
+  __device__ __forceinline__ void get(float* v, const void* lut) const {
+    const u16* const T = static_cast<const u16*>(lut);
+    uint32_t t[8], h[4];
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t w = (uint32_t)a[i];
+      t[2 * i] = lut_index(w & 0x7fffu, (w >> 15) & 1u, ok);
+      t[2 * i + 1] = lut_index((w >> 16) & 0x7fffu, w >> 31, ok);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) h[i] = (uint32_t)T[t[2 * i]] | ((uint32_t)T[t[2 * i + 1]] << 16);
+    if (__builtin_expect(!ok, 0)) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t w = (uint32_t)a[i];
+        if ((w & 0x7fffu) - kLutLo >= kLutN || ((w >> 16) & 0x7fffu) - kLutLo >= kLutN) h[i] = gelu_pair_plain(w);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __uint_as_float(h[i] << 16);
+      v[2 * i + 1] = __uint_as_float(h[i] & 0xffff0000u);
+    }
+  }
 };
 template <>
 struct Raw8<GELUB> {
@@ -173,17 +249,44 @@ struct Raw8<GELUB> {
     float x[8], g[8];
     unpack8(a, x);
     unpack8(d, g);
-    auto grad = [](float xv, float gv) {
-      float e;  // exp(-x^2 / 2)
-      const float cdf = gelu_phi(xv, &e);
-      const float pdf = 0.39894228040143267794f * e;
-      return gv * (cdf + xv * pdf);
-    };
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
-      const uint32_t h = pack_bf16x2(grad(x[i], g[i]), grad(x[i + 1], g[i + 1]));
+      const uint32_t h = pack_bf16x2(g[i] * gelu_grad_factor(x[i]), g[i + 1] * gelu_grad_factor(x[i + 1]));
       v[i] = __uint_as_float(h << 16);
       v[i + 1] = __uint_as_float(h & 0xffff0000u);
+    }
+  }
+  // the same values with the factor from the table (a copy of g_gelub_lut in LDS), read like the forward's
+  __device__ __forceinline__ void get(float* v, const void* lut) const {
+    const float* const T = static_cast<const float*>(lut);
+    uint32_t t[8], h[4];
+    float f[8];
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t w = (uint32_t)a[i];
+      t[2 * i] = lut_index(w & 0x7fffu, (w >> 15) & 1u, ok);
+      t[2 * i + 1] = lut_index((w >> 16) & 0x7fffu, w >> 31, ok);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) f[i] = T[t[i]];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t gw = (uint32_t)d[i];
+      h[i] = pack_bf16x2(__uint_as_float(gw << 16) * f[2 * i], __uint_as_float(gw & 0xffff0000u) * f[2 * i + 1]);
+    }
+    if (__builtin_expect(!ok, 0)) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t w = (uint32_t)a[i];
+        if ((w & 0x7fffu) - kLutLo >= kLutN || ((w >> 16) & 0x7fffu) - kLutLo >= kLutN)
+          h[i] = gelu_grad_pair_plain(w, (uint32_t)d[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __uint_as_float(h[i] << 16);
+      v[2 * i + 1] = __uint_as_float(h[i] & 0xffff0000u);
     }
   }
 };
@@ -369,7 +472,7 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
                                           int mvalid, int pt, int kc, uint8_t* __restrict__ q, float* __restrict__ s,
                                           uint8_t* __restrict__ q_t, float* __restrict__ s_t, uint32_t ld_t, int blocked,
                                           float eps, int64_t gate_off, u16* __restrict__ h_out, uint8_t* tile_t,
-                                          Divider* cdiv, const uint32_t* src_row = nullptr) {
+                                          Divider* cdiv, const uint32_t* src_row = nullptr, const void* lut = nullptr) {
   const bool plain_div = !kBf16Values<IN> || eps != 0.f;  // see make_scale
   float (*part)[kTile] = reinterpret_cast<float (*)[kTile]>(tile_t);
   const int64_t cols = (int64_t)nt * kTile;
@@ -410,8 +513,12 @@ __device__ __forceinline__ void dual_tile(const typename IN::elem* __restrict__ 
     const bool live = FULL || (int)r < mvalid;
     float (&vi)[8] = v[kPacked ? 0 : i];
     // (a row is unpacked where its turn comes: hoisted to the top, the rows of the whole tile would be live unpacked)
-    if constexpr (kPacked) raw[i].pin();
-    raw[i].get(vi);
+    if constexpr (kPacked) {
+      raw[i].pin();
+      raw[i].get(vi, lut);  // the activation from its table in LDS
+    } else {
+      raw[i].get(vi);
+    }
     if constexpr (kPacked) {
       const v4i pk = pack8_bf16(vi);
 #pragma unroll
@@ -479,6 +586,13 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   static_assert(sizeof(float) * 16 * kTile <= sizeof(tile_t), "the column maxima fit in the staging region");
   __shared__ Divider cdiv[kTile];  // scale and divider of every column of the tile
   __shared__ int slot;
+  // the activation's table (GELU forms only), copied from the library's array; find_group's barriers order the
+  // copy before the tile's reads
+  __shared__ __attribute__((aligned(16))) uint8_t lut_s[kLutBytes<IN> ? kLutBytes<IN> : 16];
+  if constexpr (kLutBytes<IN> != 0) {
+    const v4i* const src = reinterpret_cast<const v4i*>(std::is_same<IN, GELU>::value ? (const void*)g_gelu_lut : (const void*)g_gelub_lut);
+    for (uint32_t i = threadIdx.x; i < kLutBytes<IN> / 16; i += 256) reinterpret_cast<v4i*>(lut_s)[i] = src[i];
+  }
 
   // Workgroups go to the eight XCDs in turn, and the row-wise scales of a tile are 128 single floats, one
   // per row: with tile = workgroup index, the eight floats of a 32-byte sector would come from eight
@@ -501,9 +615,9 @@ __global__ __launch_bounds__(256) void quant_dual_grouped_kernel(
   const int64_t left = goff[g + 1] - m0;
   const int mvalid = left < kTile ? (int)left : kTile;
   if (mvalid == kTile)
-    dual_tile<IN, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, gate_off, h_out, tile_t, cdiv);
+    dual_tile<IN, true>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, gate_off, h_out, tile_t, cdiv, nullptr, lut_s);
   else
-    dual_tile<IN, false>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, gate_off, h_out, tile_t, cdiv);
+    dual_tile<IN, false>(x, (uint32_t)ldx, nt, m0, mvalid, pt, kc, q, s, q_t, s_t, (uint32_t)ld_t, blocked, eps, gate_off, h_out, tile_t, cdiv, nullptr, lut_s);
 }
 
 // The dual quantiser with the token permute fused in: x holds the tokens in their original order, and permuted
@@ -558,6 +672,20 @@ __global__ __launch_bounds__(256) void quant_dual_gather_kernel(
 // and dh and one sigmoid per position.
 // Thread (gr = tid / 16, c = tid % 16) holds rows gr*4 .. gr*4+3, columns c*8 .. c*8+7 of both tiles.
 // ---------------------------------------------------------------------------------------
+// sigmoid(a) in fp32 per bf16 value a, for |a| in [2^-14, 2^4), read from LDS like the GELU tables (filled ahead of
+// every launch by the kernel's own sigmoid; inside the table range a sigmoid(a) equals the scaled form's silu bit
+// for bit: neither product leaves the normal range there)
+constexpr uint32_t kSigLo = (uint32_t)(127 - 14) << 7;
+constexpr uint32_t kSigN = (uint32_t)(14 + 4) << 7;
+static __device__ __attribute__((aligned(16))) float g_sigmoid_lut[2 * kSigN];
+__global__ __launch_bounds__(256) void sigmoid_lut_kernel() {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= 2 * kSigN) return;
+  const uint32_t sign = i >= kSigN ? 1u : 0u;
+  const float x = __uint_as_float(((sign << 15) | (kSigLo + i - sign * kSigN)) << 16);
+  g_sigmoid_lut[i] = sigmoid_scaled(x) * 0x1p-16f;
+}
+
 // 4 values / one scale -> 4 codes in one dword
 __device__ __forceinline__ int quant4(const float* v, const Divider& d) {
   float t[4];
@@ -578,7 +706,7 @@ __device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa 
                                                      float* __restrict__ s, uint8_t* __restrict__ q_t,
                                                      float* __restrict__ s_t, uint32_t ld_t, int blocked,
                                                      u16* __restrict__ g_out, uint8_t (*tile_t)[kTile * kTLd],
-                                                     Divider (*cdiv)[kTile]) {
+                                                     Divider (*cdiv)[kTile], const float* sig_lut) {
   const int tid = threadIdx.x, gr = tid >> 4, c = tid & 15;
   const int half = nt / 2;
   const int64_t cols = (int64_t)nt * kTile;
@@ -613,17 +741,44 @@ __device__ __forceinline__ void swiglu_bwd_dual_tile(const u16* __restrict__ xa 
     unpack8(ra[i], fa);
     unpack8(rb[i], fb);
     unpack8(rd[i], fd);
+    // sigmoid(a) of the row's eight values from the table, all reads issued together; silu = a sigmoid(a)
+    float sg[8], sil[8];
+    {
+      uint32_t t[8];
+      bool ok = true;
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const uint32_t w = (uint32_t)ra[i][k];
+        const uint32_t m0 = (w & 0x7fffu) - kSigLo, m1 = ((w >> 16) & 0x7fffu) - kSigLo;
+        ok = ok && m0 < kSigN && m1 < kSigN;
+        t[2 * k] = m0 < kSigN ? m0 + ((w >> 15) & 1u) * kSigN : 0u;
+        t[2 * k + 1] = m1 < kSigN ? m1 + (w >> 31) * kSigN : 0u;
+      }
+#pragma unroll
+      for (int k = 0; k < 8; k++) sg[k] = sig_lut[t[k]];
+#pragma unroll
+      for (int k = 0; k < 8; k++) sil[k] = fa[k] * sg[k];
+      if (__builtin_expect(!ok, 0)) {  // values outside the table (zeros, outliers): the arithmetic
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+          if ((__float_as_uint(fa[k]) >> 16 & 0x7fffu) - kSigLo >= kSigN) {
+            const float rs = sigmoid_scaled(fa[k]);
+            sg[k] = rs * 0x1p-16f;
+            sil[k] = silu_from(fa[k], rs);
+          }
+        }
+      }
+    }
 #pragma unroll
     for (int k = 0; k < 8; k += 2) {
-      const float rs0 = sigmoid_scaled(fa[k]), rs1 = sigmoid_scaled(fa[k + 1]);
       // db = bf16(dh * bf16(silu(a)))
-      const uint32_t sl = pack_bf16x2(silu_from(fa[k], rs0), silu_from(fa[k + 1], rs1));
+      const uint32_t sl = pack_bf16x2(sil[k], sil[k + 1]);
       const uint32_t ob = pack_bf16x2(fd[k] * __uint_as_float(sl << 16), fd[k + 1] * __uint_as_float(sl & 0xffff0000u));
       vp[1][i][k / 2] = ob;
       v[1][k] = __uint_as_float(ob << 16);
       v[1][k + 1] = __uint_as_float(ob & 0xffff0000u);
       // da = bf16(bf16(dh * b) * sig(a) * (1 + a * (1 - sig(a))))
-      const float sg0 = rs0 * 0x1p-16f, sg1 = rs1 * 0x1p-16f;
+      const float sg0 = sg[k], sg1 = sg[k + 1];
       const uint32_t gb = pack_bf16x2(fd[k] * fb[k], fd[k + 1] * fb[k + 1]);
       const uint32_t oa = pack_bf16x2((__uint_as_float(gb << 16) * sg0) * (1.0f + fa[k] * (1.0f - sg0)),
                                       (__uint_as_float(gb & 0xffff0000u) * sg1) * (1.0f + fa[k + 1] * (1.0f - sg1)));
@@ -705,6 +860,9 @@ __global__ __launch_bounds__(512, 4) void swiglu_bwd_dual_kernel(const u16* __re
   __shared__ __attribute__((aligned(16))) uint8_t tile_ts[2][kTile * kTLd];
   __shared__ Divider cdivs[2][kTile];
   __shared__ int slot;
+  __shared__ __attribute__((aligned(16))) float sig_s[2 * kSigN];  // find_group's barriers order the copy before its reads
+  for (uint32_t i = threadIdx.x; i < 2 * kSigN / 4; i += 512)
+    reinterpret_cast<v4i*>(sig_s)[i] = reinterpret_cast<const v4i*>(g_sigmoid_lut)[i];
   // consecutive workgroups of one XCD take the eight consecutive feature tiles of a scale sector
   // (see quant_dual_grouped_kernel)
   uint32_t bx = blockIdx.x, by = blockIdx.y;
@@ -727,10 +885,10 @@ __global__ __launch_bounds__(512, 4) void swiglu_bwd_dual_kernel(const u16* __re
   const u16* const xd = dh + m0 * ld_dh + (int64_t)f * kTile;
   if (mvalid == kTile)
     swiglu_bwd_dual_tile<true>(xa, (uint32_t)ld, gate_off, xd, (uint32_t)ld_dh, nt, m0, mvalid, pt, f, q, s, q_t, s_t,
-                               (uint32_t)ld_t, blocked, g_out, tile_ts, cdivs);
+                               (uint32_t)ld_t, blocked, g_out, tile_ts, cdivs, sig_s);
   else
     swiglu_bwd_dual_tile<false>(xa, (uint32_t)ld, gate_off, xd, (uint32_t)ld_dh, nt, m0, mvalid, pt, f, q, s, q_t, s_t,
-                                (uint32_t)ld_t, blocked, g_out, tile_ts, cdivs);
+                                (uint32_t)ld_t, blocked, g_out, tile_ts, cdivs, sig_s);
 }
 
 // The 8x8 byte matrix held as eight rows of two dwords, transposed with byte permutes: cols[j]
@@ -1068,6 +1226,7 @@ extern "C" int aamd_gelu_quant_1x128_dual_grouped(const void* x, const void* dh,
   int rc = launch_group_tile_offsets(group_offsets, E, kTile, tile_ws, st);
   if (rc) return rc;
   dim3 grid((unsigned)(F / kTile), (unsigned)grid_tiles), block(256);
+  gelu_lut_kernel<<<dim3((2 * kLutN + 255) / 256), dim3(256), 0, st>>>();
   if (dh == nullptr) {
     quant_dual_grouped_kernel<GELU><<<grid, block, 0, st>>>((const u16*)x, ld, (int)(F / kTile), group_offsets, tile_ws, E, q, s,
                                                             q_t, s_t, ld_t, q_t_layout, 0.f, 0, (u16*)h_out);
@@ -1107,6 +1266,7 @@ extern "C" int aamd_swiglu_bwd_quant_1x128_dual_grouped(const void* dh, int64_t 
   if (rc) return rc;
   const int nt = (int)(2 * F / kTile);
   dim3 grid((unsigned)(nt / 2), (unsigned)grid_tiles), block(512);  // two teams: the da and the db tile of a feature tile
+  sigmoid_lut_kernel<<<dim3((2 * kSigN + 255) / 256), dim3(256), 0, st>>>();
   swiglu_bwd_dual_kernel<<<grid, block, 0, st>>>((const u16*)fc1, ld, F, (const u16*)dh, ld_dh, nt, group_offsets, tile_ws, E,
                                                  q, s, q_t, s_t, ld_t, q_t_layout, (u16*)g_out);
   AAMD_LAUNCH_CHECK("swiglu_bwd_quant_dual_grouped");
