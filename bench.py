@@ -505,7 +505,29 @@ def run_gemm(args, kernels, dev, workload=None, steps=None, warmup=None, cpu_bas
         wg_med = statistics.median([sum(wg_timer.ms()[i * n_wg : (i + 1) * n_wg]) / n_wg for i in range(steps)])
         extras["wgrad_kernel"] = {"avg_launch_ms": round(wg_avg, 4), "median_launch_ms": round(wg_med, 4),
                                   "achieved_tflops": round(wg_flops / (wg_avg * 1e-3) / 1e12, 2),
-                                  "frac": round(wg_flops / (wg_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
+                                  "frac": round(wg_flops / (wg_avg * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4),
+                                  "output": "fp32 (a main_grad buffer)"}
+        if not args.no_extras:
+            # the same launches writing bf16, the dtype of the parameters, beside fp32: each launch repeated back to
+            # back (five timed after two untimed), which at the power cap runs a few per cent slower than inside
+            # the step, where the launches around it draw less
+            b2b = {}
+            for name, dt in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+                t = Timer()
+                for L in layers:
+                    dw = torch.empty((L.E, L.N, L.K), dtype=dt, device=dev)
+                    for i in range(7):
+                        a, b = t.region() if i >= 2 else (None, None)
+                        if a is not None:
+                            a.record()
+                        kernels.grouped_gemm_wgrad(L.qdy_t, L.sdy_t, L.qx_t, L.sx_t, L.goff, out=dw)
+                        if b is not None:
+                            b.record()
+                    del dw
+                torch.cuda.synchronize()
+                b2b[name] = {"avg_launch_ms": round(t.mean(), 4),
+                             "frac": round(wg_flops / (t.mean() * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
+            extras["wgrad_kernel"]["back_to_back_by_output_dtype"] = b2b
 
     if workload == "c2" and probes and not args.no_extras and args.operands == "random":
         extras["forward_gemm_by_operand_data"] = operand_data_probe(kernels, layers[0], dev)
