@@ -267,3 +267,25 @@ def test_patch_grouped_linear_hook():
     assert ns.GroupedLinear is ATorchGroupedLinear and ns.ATorchGroupedLinear is ATorchGroupedLinear
     assert not hasattr(ns, "_ATorchQuantizedGroupedLinear")
     patch_grouped_linear(None)
+
+
+def test_layouts_of_the_transposed_codes_on_the_host():
+    """The token-block-major layout [ld_t/128, R, 128] holds byte (r, t) at ((t / 128) R + r) 128 + t % 128;
+    ``qt_rows`` turns it into the row layout [R, ld_t] and ``qt_ld`` reads the padded token count of either."""
+    from atorch_amd import kernels
+
+    R, ld_t = 5, 384
+    rows = torch.arange(R * ld_t, dtype=torch.int64).remainder(251).to(torch.uint8).view(R, ld_t)
+    blocked = torch.empty(ld_t // TILE * R * TILE, dtype=torch.uint8)
+    for r in range(R):
+        for t in range(0, ld_t, 37):
+            blocked[((t // TILE) * R + r) * TILE + t % TILE] = rows[r, t]
+    blocked = blocked.view(ld_t // TILE, R, TILE)
+    back = kernels.qt_rows(blocked)
+    assert back.shape == (R, ld_t) and kernels.qt_ld(blocked) == ld_t and kernels.qt_ld(rows) == ld_t
+    for r in range(R):
+        for t in range(0, ld_t, 37):
+            assert back[r, t] == rows[r, t]
+    assert kernels.qt_rows(rows) is rows
+    assert kernels._alloc_qt(R, ld_t, True, "cpu").shape == (ld_t // TILE, R, TILE)
+    assert kernels._alloc_qt(R, ld_t, False, "cpu").shape == (R, ld_t)
