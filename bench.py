@@ -68,7 +68,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "quant"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "quant", "module"],
                     help="c1-c5: the configurations of the benchmark; quant: every quantisation kernel of the path at "
                          "the c2 shapes, each beside the streaming probe of its read:write mix")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -877,6 +877,16 @@ def main():
         mixes = MIXES if args.mix_probe == "all" else args.mix_probe.split(",")
         print(json.dumps({"metric": "streaming probe GB/s by read:write mix", "unit": "GB/s", "n_gpus": 1,
                           "mixes": mix_probe(dev, mixes)}))  # fmt: skip
+        return
+    if args.workload == "module":
+        # the expert MLP through the Python mirror alone (what extras.module_step of the default run reports): the
+        # run a kernel trace of the whole forward + backward is taken from
+        ms = module_step(kernels, dev, steps=args.steps)
+        c = ms["cached_weight_codes"]
+        print(json.dumps({"metric": "fp8 expert MLP forward + backward TFLOPS (module level)", "value": c["TFLOP/s"],
+                          "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": 2, "ms_per_step": c["ms_per_step"],
+                          "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8",
+                          "data": "synthetic", "config": {"workload": ms["what"]}, "extras": ms}))  # fmt: skip
         return
     if args.workload == "quant":
         res = run_quant(args, kernels, dev)
