@@ -57,13 +57,67 @@ def reset_wgrad_if_needed(ctx, weight: torch.Tensor, wgrad: Optional[torch.Tenso
     return None
 
 
+def _quantize_groups(op, rows: torch.Tensor, m_splits: List[int], qparams, want_transpose: bool):
+    """1x128 codes of the row groups of ``rows`` as four per-group lists (codes, scales and, with
+    ``want_transpose``, the codes and scales quantised along the tokens; else two empty lists): one launch where the
+    operator offers the fused form, the reference's loop over the groups (quantized_grouped_linear.py:90-101,
+    200-206) otherwise."""
+    if getattr(op, "supports_fused_grouped", False):
+        return op.quantize_grouped(rows, m_splits, qparams, return_transpose=want_transpose)
+    results = [op.quantize(part, qparams, return_transpose=want_transpose) for part in torch.split(rows, m_splits)]
+    transposed = results if want_transpose else []
+    return ([r.data for r in results], [r.scale for r in results],
+            [r.data_t for r in transposed], [r.scale_t for r in transposed])  # fmt: skip
+
+
+def _weight_codes(op, weights, caches, qlinear_params, is_first_microbatch, want_transpose: bool):
+    """Block-quantised weights as four per-expert lists, under the caching rule of
+    quantized_grouped_linear.py:103-134: quantise on the first microbatch (True or None), when
+    FORCE_QUANTIZE_PER_MICROBATCH is set, or when a backward needs transposes the caches do not hold; otherwise
+    serve the caches.  Fresh codes are written back to the caches unless the environment flag forces
+    quantisation anyway."""
+    forced = force_quantize_per_microbatch()
+    first = is_first_microbatch or is_first_microbatch is None
+    stale = want_transpose and caches[0].data_t is None
+    if not (forced or first or stale):
+        held = [c.to_qresult() for c in caches]
+        transposed = held if want_transpose else []
+        return ([r.data for r in held], [r.scale for r in held],
+                [r.data_t for r in transposed], [r.scale_t for r in transposed])  # fmt: skip
+    if getattr(op, "supports_fused_grouped", False):
+        q, s, q_t, s_t = op.quantize_weights(weights, qlinear_params.w_params, return_transpose=want_transpose)
+    else:
+        fresh = [op.quantize(w, qlinear_params.w_params, return_transpose=want_transpose) for w in weights]
+        transposed = fresh if want_transpose else []
+        q, s = [r.data for r in fresh], [r.scale for r in fresh]
+        q_t, s_t = [r.data_t for r in transposed], [r.scale_t for r in transposed]
+    if not forced:
+        for i, cache in enumerate(caches):
+            cache.data, cache.scale = q[i], s[i]
+            cache.data_t = q_t[i] if want_transpose else None
+            cache.scale_t = s_t[i] if want_transpose else None
+    return q, s, q_t, s_t
+
+
+def _adds_to_main_grad(fuse_wgrad_accumulation: bool, is_first_microbatch) -> bool:
+    """Does this backward add to ``main_grad`` (True) or overwrite it?  quantized_grouped_linear.py:232-235: with
+    fused accumulation every microbatch but the one flagged first adds; an unflagged call (None) adds."""
+    return bool(fuse_wgrad_accumulation and not (is_first_microbatch is not None and is_first_microbatch))
+
+
 class _ATorchQuantizedGroupedLinear(torch.autograd.Function):
     """Grouped linear with 1x128 / 128x128 fp8 quantisation.
 
     fwd   : Y_g  = X_g W_g^T (+ b_g)
     dgrad : dX_g = dY_g W_g
     wgrad : dW_g = dY_g^T X_g
+
+    Argument order and the gradient tuple are those of the reference's function
+    (quantized_grouped_linear.py:51-71, 257-270); the work between them goes through the operator object's
+    list-of-groups interface, fused where it can be.
     """
+
+    NUM_NON_TENSOR_ARGS = 9  # m_splits .. fuse_wgrad_accumulation: a None each in the gradient tuple
 
     @staticmethod
     def forward(  # type: ignore
@@ -80,185 +134,69 @@ class _ATorchQuantizedGroupedLinear(torch.autograd.Function):
         fuse_wgrad_accumulation: bool,
         *weights_and_biases: torch.Tensor,
     ) -> torch.Tensor:
-        assert qlinear_params.quantize_op is not None
-        quantize_op = qlinear_params.quantize_op
-        fused = bool(getattr(quantize_op, "supports_fused_grouped", False))
-
+        op = qlinear_params.quantize_op
+        assert op is not None
         num_gemms = len(m_splits)
-        weights = weights_and_biases[:num_gemms]
-        biases = list(weights_and_biases[num_gemms:])
-        device = x.device
-
-        x_shape = x.shape
-        out_dtype = x.dtype if qlinear_params.mm_fprop.out_dtype is None else qlinear_params.mm_fprop.out_dtype
-        in_features = weights[0].shape[-1]
-        assert x_shape[-1] == in_features, "GEMM not possible"
-        x2d = x.view(-1, in_features)
+        weights, biases = weights_and_biases[:num_gemms], list(weights_and_biases[num_gemms:])
+        out_features, in_features = weights[0].shape
+        assert x.shape[-1] == in_features, "GEMM not possible"
         if use_bias:
             assert len(biases) == num_gemms, "Number of biases should match number of GEMMs."
             biases = [cast_if_needed(b, activation_dtype) for b in biases]
+        rows = x.view(-1, in_features)
 
-        # Quantize x (with optional transpose).
-        if fused:
-            qx_list, sx_list, qx_t_list, sx_t_list = quantize_op.quantize_grouped(
-                x2d, m_splits, qlinear_params.x_params, return_transpose=is_grad_enabled
-            )
-        else:
-            qx_list, sx_list, qx_t_list, sx_t_list = [], [], [], []
-            for x_i in torch.split(x2d, m_splits):
-                r = quantize_op.quantize(x_i, qlinear_params.x_params, return_transpose=is_grad_enabled)
-                qx_list.append(r.data)
-                sx_list.append(r.scale)
-                if is_grad_enabled:
-                    qx_t_list.append(r.data_t)
-                    sx_t_list.append(r.scale_t)
+        qx, sx, qx_t, sx_t = _quantize_groups(op, rows, m_splits, qlinear_params.x_params, is_grad_enabled)
+        qw, sw, qw_t, sw_t = _weight_codes(op, weights, weight_qresult_caches, qlinear_params, is_first_microbatch,
+                                           is_grad_enabled)  # fmt: skip
 
-        # Quantize w only when is_first_microbatch is True or None (or the cache cannot serve).
-        qw_list, sw_list, qw_t_list, sw_t_list = [], [], [], []
-        update_fp8_weights = is_first_microbatch or is_first_microbatch is None
-        force = force_quantize_per_microbatch()
-        if force or update_fp8_weights or (is_grad_enabled and weight_qresult_caches[0].data_t is None):
-            if fused:
-                qw_list, sw_list, qw_t_list, sw_t_list = quantize_op.quantize_weights(
-                    weights, qlinear_params.w_params, return_transpose=is_grad_enabled
-                )
-            else:
-                for w in weights:
-                    r = quantize_op.quantize(w, qlinear_params.w_params, return_transpose=is_grad_enabled)
-                    qw_list.append(r.data)
-                    sw_list.append(r.scale)
-                    if is_grad_enabled:
-                        qw_t_list.append(r.data_t)
-                        sw_t_list.append(r.scale_t)
-            if not force:
-                for i, cache in enumerate(weight_qresult_caches):
-                    cache.data = qw_list[i]
-                    cache.scale = sw_list[i]
-                    cache.data_t = qw_t_list[i] if is_grad_enabled else None
-                    cache.scale_t = sw_t_list[i] if is_grad_enabled else None
-        else:
-            for cache in weight_qresult_caches:
-                r = cache.to_qresult()
-                qw_list.append(r.data)
-                sw_list.append(r.scale)
-                if is_grad_enabled:
-                    qw_t_list.append(r.data_t)
-                    sw_t_list.append(r.scale_t)
-
-        out = torch.empty([sum(m_splits), weights[0].size(0)], dtype=out_dtype, device=device)
-        quantize_op.grouped_qgemm(
-            qx_list,
-            qw_list,
-            qlinear_params.mm_fprop,
-            sx_list,
-            sw_list,
-            list(torch.split(out, m_splits)),
-            bias=biases if use_bias else None,
-            qparams_x=qlinear_params.x_params,
-            qparams_w=qlinear_params.w_params,
-        )
+        y_dtype = qlinear_params.mm_fprop.out_dtype or x.dtype
+        out = torch.empty((sum(m_splits), out_features), dtype=y_dtype, device=x.device)
+        op.grouped_qgemm(qx, qw, qlinear_params.mm_fprop, sx, sw, list(torch.split(out, m_splits)),
+                         bias=biases if use_bias else None,
+                         qparams_x=qlinear_params.x_params, qparams_w=qlinear_params.w_params)  # fmt: skip
 
         if is_grad_enabled:
-            ctx.m_splits = m_splits
-            ctx.num_gemms = num_gemms
-            ctx.use_bias = use_bias
-            ctx.x_shape = x_shape
-            ctx.qlinear_params = qlinear_params
-            ctx.quantize_op = quantize_op
-            ctx.is_first_microbatch = is_first_microbatch
-            ctx.fuse_wgrad_accumulation = fuse_wgrad_accumulation
-            ctx.device = device
+            ctx.m_splits, ctx.num_gemms, ctx.use_bias, ctx.x_shape = m_splits, num_gemms, use_bias, x.shape
+            ctx.qlinear_params, ctx.quantize_op, ctx.device = qlinear_params, op, x.device
+            ctx.is_first_microbatch, ctx.fuse_wgrad_accumulation = is_first_microbatch, fuse_wgrad_accumulation
             # the Python-side attributes (main_grad, grad_added_to_main_grad) are read from
             # these references, not from the re-materialised saved tensors
             ctx.weight_refs = list(weights)
-            ctx.save_for_backward(*qx_t_list, *sx_t_list, *qw_t_list, *sw_t_list, *weights)
-
-        return out.view(-1, *x_shape[1:-1], out.shape[-1])
+            ctx.save_for_backward(*qx_t, *sx_t, *qw_t, *sw_t, *weights)
+        return out.view(-1, *x.shape[1:-1], out_features)
 
     @staticmethod
     def backward(ctx, *dy_tup: torch.Tensor) -> Tuple[Union[torch.Tensor, None], ...]:
-        assert len(dy_tup) == 1
-        dy = dy_tup[0]
-        n = ctx.num_gemms
-        qx_t_list = ctx.saved_tensors[:n]
-        sx_t_list = ctx.saved_tensors[n : 2 * n]
-        qw_t_list = ctx.saved_tensors[2 * n : 3 * n]
-        sw_t_list = ctx.saved_tensors[3 * n : 4 * n]
+        (dy,) = dy_tup
+        n, qp, op, m_splits = ctx.num_gemms, ctx.qlinear_params, ctx.quantize_op, ctx.m_splits
+        saved = ctx.saved_tensors
+        assert len(saved) == 5 * n
+        qx_t, sx_t, qw_t, sw_t = (saved[i * n : (i + 1) * n] for i in range(4))
         weights = ctx.weight_refs
-        assert len(ctx.saved_tensors) == 5 * n
-        qp = ctx.qlinear_params
-        quantize_op = ctx.quantize_op
-        fused = bool(getattr(quantize_op, "supports_fused_grouped", False))
+        out_features, in_features = weights[0].shape
 
-        out_dtype_dgrad = dy.dtype if qp.mm_dgrad.out_dtype is None else qp.mm_dgrad.out_dtype
-        dy = dy.contiguous()
-        dy = dy.view(-1, dy.shape[-1])
-        dy_list = torch.split(dy, ctx.m_splits)
+        dy_rows = dy.contiguous().view(-1, dy.shape[-1])
+        bias_grads = [part.sum(dim=0) if ctx.use_bias else None for part in torch.split(dy_rows, m_splits)]
+        qdy, sdy, qdy_t, sdy_t = _quantize_groups(op, dy_rows, m_splits, qp.g_params, True)
 
-        b_grad_list = [torch.sum(dy_i, dim=0) if ctx.use_bias else None for dy_i in dy_list]
-        if fused:
-            qdy_list, sdy_list, qdy_t_list, sdy_t_list = quantize_op.quantize_grouped(
-                dy, ctx.m_splits, qp.g_params, return_transpose=True
-            )
-        else:
-            qdy_list, sdy_list, qdy_t_list, sdy_t_list = [], [], [], []
-            for dy_i in dy_list:
-                r = quantize_op.quantize(dy_i, qp.g_params, return_transpose=True)
-                qdy_list.append(r.data)
-                sdy_list.append(r.scale)
-                qdy_t_list.append(r.data_t)
-                sdy_t_list.append(r.scale_t)
+        # dX_g = dY_g W_g
+        dgrad = torch.empty((sum(m_splits), in_features), dtype=qp.mm_dgrad.out_dtype or dy.dtype, device=ctx.device)
+        op.grouped_qgemm(qdy, qw_t, qp.mm_dgrad, sdy, sw_t, list(torch.split(dgrad, m_splits)),
+                         qparams_x=qp.g_params, qparams_w=qp.w_params)  # fmt: skip
 
-        dgrad = torch.empty((sum(ctx.m_splits), weights[0].size(1)), dtype=out_dtype_dgrad, device=ctx.device)
-        quantize_op.grouped_qgemm(
-            qdy_list,
-            qw_t_list,
-            qp.mm_dgrad,
-            sdy_list,
-            sw_t_list,
-            list(torch.split(dgrad, ctx.m_splits)),
-            qparams_x=qp.g_params,
-            qparams_w=qp.w_params,
-        )
-
-        if ctx.is_first_microbatch is not None:
-            accumulate_wgrad_into_param_main_grad = ctx.fuse_wgrad_accumulation and not ctx.is_first_microbatch
-        else:
-            accumulate_wgrad_into_param_main_grad = ctx.fuse_wgrad_accumulation
-
-        out_dtype_wgrad = dy.dtype if qp.mm_wgrad.out_dtype is None else qp.mm_wgrad.out_dtype
+        # dW_g = dY_g^T X_g, into main_grad or into a fresh buffer
         if ctx.fuse_wgrad_accumulation:
-            wgrad_list = [w.main_grad for w in weights]
+            wgrads = [w.main_grad for w in weights]
         else:
-            wbuf = torch.empty((n, *weights[0].size()), dtype=out_dtype_wgrad, device=ctx.device)
-            wgrad_list = list(wbuf.unbind(0))
-        quantize_op.grouped_qgemm(
-            qdy_t_list,
-            qx_t_list,
-            qp.mm_wgrad,
-            sdy_t_list,
-            sx_t_list,
-            wgrad_list,
-            accumulate=accumulate_wgrad_into_param_main_grad,
-            qparams_x=qp.g_params,
-            qparams_w=qp.x_params,
-        )
-        wgrad_list = [reset_wgrad_if_needed(ctx, w, wgrad) for w, wgrad in zip(weights, wgrad_list)]
+            wgrads = list(torch.empty((n, out_features, in_features), dtype=qp.mm_wgrad.out_dtype or dy.dtype,
+                                      device=ctx.device).unbind(0))  # fmt: skip
+        op.grouped_qgemm(qdy_t, qx_t, qp.mm_wgrad, sdy_t, sx_t, wgrads,
+                         accumulate=_adds_to_main_grad(ctx.fuse_wgrad_accumulation, ctx.is_first_microbatch),
+                         qparams_x=qp.g_params, qparams_w=qp.x_params)  # fmt: skip
+        wgrads = [reset_wgrad_if_needed(ctx, w, g) for w, g in zip(weights, wgrads)]
 
-        return (
-            dgrad.view(ctx.x_shape),
-            None,
-            None,
-            None,
-            None,
-            None,
-            None,
-            None,
-            None,
-            None,
-            *wgrad_list,
-            *b_grad_list,
-        )
+        nones = (None,) * _ATorchQuantizedGroupedLinear.NUM_NON_TENSOR_ARGS
+        return (dgrad.view(ctx.x_shape), *nones, *wgrads, *bias_grads)
 
 
 def _stack_of(ts) -> Optional[torch.Tensor]:
@@ -368,10 +306,7 @@ class _GroupedLinearDeviceOffsets(torch.autograd.Function):
         )
         dgrad = kernels.grouped_gemm_nt(qdy, sdy, qw_t, sw_t, goff, out_dtype=f32_if_half(dgrad_dtype)).to(dgrad_dtype)
 
-        if ctx.is_first_microbatch is not None:
-            accumulate = ctx.fuse_wgrad_accumulation and not ctx.is_first_microbatch
-        else:
-            accumulate = ctx.fuse_wgrad_accumulation
+        accumulate = _adds_to_main_grad(ctx.fuse_wgrad_accumulation, ctx.is_first_microbatch)
         if ctx.fuse_wgrad_accumulation:
             main = _stack_of([w.main_grad for w in weights])
             if main is not None and main.dtype in (torch.float32, torch.bfloat16):
