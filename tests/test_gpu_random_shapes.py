@@ -69,12 +69,14 @@ def test_grouped_gemms_on_random_shapes(seed):
         if M > 40000 or N * K * E > 32 * 1024 * 1024:
             continue
         dy = (torch.randn(M, N, device=dev) * 0.01).bfloat16()
-        _, _, qxt, sxt = kernels.tile_quant_dual_grouped(x, goff, E, rowwise=False)
-        _, _, qdt, sdt = kernels.tile_quant_dual_grouped(dy, goff, E, ld_t=qxt.shape[1], rowwise=False)
+        blocked = (seed + case) % 2 == 0  # the two layouts of the transposed codes in turn
+        _, _, qxt, sxt = kernels.tile_quant_dual_grouped(x, goff, E, rowwise=False, blocked=blocked)
+        _, _, qdt, sdt = kernels.tile_quant_dual_grouped(dy, goff, E, ld_t=kernels.qt_ld(qxt), rowwise=False, blocked=blocked)
         base = torch.randn(E, N, K, device=dev)
         acc = base.clone()
         kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out=acc, accumulate=True)
         dw = kernels.grouped_gemm_wgrad(qdt, sdt, qxt, sxt, goff, out_dtype=torch.float32)
+        qxt, qdt = kernels.qt_rows(qxt), kernels.qt_rows(qdt)  # [rows, ld_t] for the definition below
         refw = torch.zeros(E, N, K, dtype=torch.float64, device=dev)
         col = 0  # groups are padded to whole 128-token blocks along the transposed operands' columns
         for e, m in enumerate(splits):
@@ -118,12 +120,14 @@ def test_dual_quantisers_on_random_shapes(oracle, seed):
         goff = kernels.group_offsets_from_splits(splits, dev)
         ptot = oracle.padded_offsets(splits)[-1]
 
+        blocked = (seed + case) % 2 == 0  # the fused kernels write the two layouts of the transposed codes in turn
+
         def same_as_plain(res, h):
             # the fused kernel's codes and scales are those of the plain kernel on the fused kernel's own values
             q, s, q_t, s_t = res
-            q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(h, goff, E, ld_t=q_t.shape[1])
+            q2, s2, q_t2, s_t2 = kernels.tile_quant_dual_grouped(h, goff, E, ld_t=kernels.qt_ld(q_t))
             assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2), what
-            assert torch.equal(q_t.view(torch.uint8)[:, :ptot], q_t2.view(torch.uint8)[:, :ptot]), what
+            assert torch.equal(kernels.qt_rows(q_t).view(torch.uint8)[:, :ptot], q_t2.view(torch.uint8)[:, :ptot]), what
             assert torch.equal(s_t[: ptot // TILE], s_t2[: ptot // TILE]), what
 
         q, s, q_t, s_t = kernels.tile_quant_dual_grouped(x.to(dev), goff, E)
@@ -135,13 +139,13 @@ def test_dual_quantisers_on_random_shapes(oracle, seed):
 
         fc1 = torch.cat([x, (torch.randn(M, F, generator=g)).bfloat16()], dim=1).contiguous().to(dev)
         dh = (torch.randn(M, F, generator=g) * 0.1).bfloat16().to(dev)
-        *res, h = kernels.swiglu_tile_quant_dual_grouped(fc1, goff, E, return_activation=True)
+        *res, h = kernels.swiglu_tile_quant_dual_grouped(fc1, goff, E, return_activation=True, blocked=blocked)
         same_as_plain(res, h)
-        *res, h = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, E, return_activation=True)
+        *res, h = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, E, return_activation=True, blocked=blocked)
         same_as_plain(res, h)
-        *res, gx = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, E, dh=dh, return_activation=True)
+        *res, gx = kernels.gelu_tile_quant_dual_grouped(x.to(dev), goff, E, dh=dh, return_activation=True, blocked=blocked)
         same_as_plain(res, gx)
-        *res, gfc1 = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E, return_grad=True)
+        *res, gfc1 = kernels.swiglu_bwd_tile_quant_dual_grouped(dh, fc1, goff, E, return_grad=True, blocked=blocked)
         same_as_plain(res, gfc1)
         assert torch.equal(gfc1.cpu(), oracle.swiglu_bwd(dh.cpu(), fc1.cpu())) or rel_err(
             gfc1.float().cpu(), oracle.swiglu_bwd(dh.cpu(), fc1.cpu()).float()
